@@ -1,0 +1,17 @@
+"""MI355X (gfx950) implementation of BitMTP's packed low-bit GEMV hot path:
+T2-g128 ternary and Q1-g128 sign weights times per-token INT8 activations."""
+from . import contracts  # noqa: F401
+from .ops import (  # noqa: F401
+    OUT_BF16, OUT_F32, OUT_G32,
+    init_kernels, load_actq_kernel, load_q1_kernel, load_t2_kernel,
+    packed_gemv_ex, packed_int8_linear, q1g128_int8xint1_linear, q1g128_w1a16_linear,
+    quant_input, t2g128_int8xint2_linear,
+)
+from .packing import pack_q1_g128, pack_t2_g128, unpack_q1_g128, unpack_t2_g128  # noqa: F401
+
+__all__ = [
+    "contracts", "init_kernels", "load_actq_kernel", "load_q1_kernel", "load_t2_kernel",
+    "packed_gemv_ex", "packed_int8_linear", "q1g128_int8xint1_linear", "q1g128_w1a16_linear",
+    "quant_input", "t2g128_int8xint2_linear", "pack_q1_g128", "pack_t2_g128",
+    "unpack_q1_g128", "unpack_t2_g128", "OUT_BF16", "OUT_F32", "OUT_G32",
+]

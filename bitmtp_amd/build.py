@@ -1,0 +1,75 @@
+"""Builds the gfx950 shared libraries of this package with hipcc, in-tree.
+
+    python -m bitmtp_amd.build            # build what is missing or out of date
+    python -m bitmtp_amd.build --force    # rebuild everything
+
+The libraries keep the file names the reference loader expects
+(``t2g128_kernels/libbonsai_t2.so`` and ``q1g128_kernels/libbonsai_q1.so`` next
+to the operator module, src/bonsai_sft/gpu/model.py:77-78,209-210; its build
+script is src/bonsai_sft/gpu/t2g128_kernels/compile.sh:12-18).  hipcc
+cross-compiles for gfx950 without a GPU.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+
+# source (under csrc/) -> library (under the package)
+TARGETS = {
+    "t2g128_kernels.hip": os.path.join("t2g128_kernels", "libbonsai_t2.so"),
+    "q1g128_kernels.hip": os.path.join("q1g128_kernels", "libbonsai_q1.so"),
+    "act_quant.hip": os.path.join("act_quant", "libbonsai_actq.so"),
+}
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed fp32 VALU forms are kept out of generated code on this target
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def lib_path(source: str) -> str:
+    return os.path.join(HERE, TARGETS[source])
+
+
+def _deps() -> list[str]:
+    return [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [
+        os.path.join(HERE, "..", "include", "bonsai_gemv.h")]
+
+
+def _stale(out: str) -> bool:
+    if not os.path.exists(out):
+        return True
+    t = os.path.getmtime(out)
+    return any(os.path.getmtime(d) > t for d in _deps() if os.path.exists(d))
+
+
+def _build_one(source: str) -> str:
+    out = lib_path(source)
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    cmd = [hipcc] + HIPCC_FLAGS + [os.path.join(CSRC, source), "-o", out]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {source}:\n{proc.stdout}")
+    return out
+
+
+def build_all(force: bool = False, verbose: bool = True) -> list[str]:
+    todo = [s for s in TARGETS if os.path.exists(os.path.join(CSRC, s))
+            and (force or _stale(lib_path(s)))]
+    with ThreadPoolExecutor(max_workers=max(1, len(todo))) as pool:
+        built = list(pool.map(_build_one, todo))
+    if verbose:
+        for b in built:
+            print(f"[bitmtp_amd.build] built {os.path.relpath(b, HERE)}")
+    return [lib_path(s) for s in TARGETS if os.path.exists(lib_path(s))]
+
+
+if __name__ == "__main__":
+    build_all(force="--force" in sys.argv[1:])

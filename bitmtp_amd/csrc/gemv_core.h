@@ -1,0 +1,182 @@
+// Per-lane arithmetic of the packed low-bit GEMV kernels.
+//
+// Everything here is plain integer code that compiles both as gfx950 device
+// code (included by packed_gemv.hip.h) and as host C++ (included by the lane
+// simulator under tests/host_sim/, which replays the exact staging layout and
+// unpack/dot sequence on the CPU so that index mistakes are found without a GPU).
+//
+// Work decomposition.  A weight row is cut into 16-byte CHUNKS (one
+// global_load_dwordx4 per lane): 64 weights for T2 (half a scale group), 128
+// for Q1 (one scale group).  A packed dword p is turned into byte vectors with
+// the cheapest possible sequence,
+//     T2:  u_j = (p >> 2j) & 0x03030303   j = 0..3   byte b of u_j = code of weight 4b + j
+//     Q1:  u_j = (p >>  j) & 0x01010101   j = 0..7   byte b of u_j = bit  of weight 8b + j
+// i.e. the codes/bits are used as they are (0..3 / 0..1) and in an interleaved
+// K order.  Both departures from the natural layout are paid for once per
+// token, when the activations are staged:
+//   * the activations are stored pre-permuted, so that dword j of an activation
+//     unit lines up with u_j (a 4x4 byte transpose of the natural order), and
+//   * the code offset is removed with the per-chunk activation sum:
+//         T2:  sum a*(code-2)  = sum a*code - 2*asum
+//         Q1:  sum a*(2*bit-1) = 2*sum a*bit - asum
+// An integer dot product does not depend on the order of its terms, so the
+// int32 group sums stay exact.
+//
+// Reference arithmetic being reproduced:
+//   src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:21-27,62-81
+//   src/bonsai_sft/gpu/q1g128_kernels/q1g128_kernels.h:47-68,388-410
+#ifndef BONSAI_GEMV_CORE_H
+#define BONSAI_GEMV_CORE_H
+
+#include <stdint.h>
+
+#if defined(__HIP_DEVICE_COMPILE__) || defined(__HIPCC__)
+#define BONSAI_HD __host__ __device__ __forceinline__
+#else
+#define BONSAI_HD inline
+#endif
+
+namespace bonsai {
+
+struct alignas(16) u32x4 {
+    uint32_t x, y, z, w;
+};
+
+// Signed 4 x int8 dot product with int32 accumulate (v_dot4_i32_i8 on gfx950).
+BONSAI_HD int dot4_i8(uint32_t a, uint32_t b, int acc) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_sdot4((int)a, (int)b, acc, false);
+#else
+    for (int i = 0; i < 4; ++i)
+        acc += (int)(int8_t)(a >> (8 * i)) * (int)(int8_t)(b >> (8 * i));
+    return acc;
+#endif
+}
+
+template <int BITS>
+struct Fmt;
+
+template <>
+struct Fmt<2> {
+    static constexpr int kChunkWeights = 64;  // weights in one 16-byte chunk
+    static constexpr int kUnits = 4;          // 16-byte activation units per chunk
+    static constexpr int kUnitsPerDword = 1;  // activation units consumed per packed dword
+    static constexpr int kVecPerDword = 4;    // byte vectors unpacked from one packed dword
+    static constexpr int kGroupShift = 1;     // scale group = chunk >> kGroupShift
+};
+
+template <>
+struct Fmt<1> {
+    static constexpr int kChunkWeights = 128;
+    static constexpr int kUnits = 8;
+    static constexpr int kUnitsPerDword = 2;
+    static constexpr int kVecPerDword = 8;
+    static constexpr int kGroupShift = 0;
+};
+
+// out[d].byte[b] = in[b].byte[d]
+BONSAI_HD u32x4 transpose4x4_bytes(uint32_t i0, uint32_t i1, uint32_t i2, uint32_t i3) {
+    u32x4 o;
+    o.x = (i0 & 0xffu) | ((i1 & 0xffu) << 8) | ((i2 & 0xffu) << 16) | ((i3 & 0xffu) << 24);
+    o.y = ((i0 >> 8) & 0xffu) | (((i1 >> 8) & 0xffu) << 8) | (((i2 >> 8) & 0xffu) << 16) |
+          (((i3 >> 8) & 0xffu) << 24);
+    o.z = ((i0 >> 16) & 0xffu) | (((i1 >> 16) & 0xffu) << 8) | (((i2 >> 16) & 0xffu) << 16) |
+          (((i3 >> 16) & 0xffu) << 24);
+    o.w = (i0 >> 24) | ((i1 >> 24) << 8) | ((i2 >> 24) << 16) | ((i3 >> 24) << 24);
+    return o;
+}
+
+BONSAI_HD int sum4_i8(uint32_t a) { return dot4_i8(a, 0x01010101u, 0); }
+
+// Index of activation unit `unit` of chunk `chunk` for tile token `m` in the
+// staged array (16-byte elements).  Units are the slow index so that the lanes
+// of a wave, which hold consecutive chunks, read consecutive 16-byte words.
+template <int BITS>
+BONSAI_HD int act_index(int m, int unit, int chunk, int chunks_per_row) {
+    return (m * Fmt<BITS>::kUnits + unit) * chunks_per_row + chunk;
+}
+
+// Stage one chunk of one token: `src` points at the chunk's kChunkWeights
+// natural-order int8 activations (16-byte aligned); writes kUnits permuted
+// units into act[] and returns the sum of the chunk's activations.
+template <int BITS>
+BONSAI_HD int stage_chunk(const u32x4 *src, u32x4 *act, int m, int chunk, int chunks_per_row) {
+    int sum = 0;
+    if (BITS == 2) {
+        for (int t = 0; t < 4; ++t) {
+            u32x4 in = src[t];  // activations 16t .. 16t+15
+            sum += sum4_i8(in.x) + sum4_i8(in.y) + sum4_i8(in.z) + sum4_i8(in.w);
+            // unit t, dword j, byte b  <-  activation 16t + 4b + j
+            act[act_index<BITS>(m, t, chunk, chunks_per_row)] =
+                transpose4x4_bytes(in.x, in.y, in.z, in.w);
+        }
+    } else {
+        for (int t = 0; t < 4; ++t) {
+            u32x4 lo = src[2 * t], hi = src[2 * t + 1];  // activations 32t .. 32t+31
+            sum += sum4_i8(lo.x) + sum4_i8(lo.y) + sum4_i8(lo.z) + sum4_i8(lo.w);
+            sum += sum4_i8(hi.x) + sum4_i8(hi.y) + sum4_i8(hi.z) + sum4_i8(hi.w);
+            // unit 2t+h, dword d, byte b  <-  activation 32t + 8b + 4h + d
+            act[act_index<BITS>(m, 2 * t, chunk, chunks_per_row)] =
+                transpose4x4_bytes(lo.x, lo.z, hi.x, hi.z);
+            act[act_index<BITS>(m, 2 * t + 1, chunk, chunks_per_row)] =
+                transpose4x4_bytes(lo.y, lo.w, hi.y, hi.w);
+        }
+    }
+    return sum;
+}
+
+// Raw dot products of one 16-byte weight chunk against MT staged tokens:
+// raw[m] += sum_k a[m][k] * code[k] (codes 0..3 for T2, bits 0..1 for Q1).
+template <int BITS, int MT>
+BONSAI_HD void chunk_dot_raw(const u32x4 w, const u32x4 *act, int chunk, int chunks_per_row,
+                             int raw[MT]) {
+    const uint32_t p[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (BITS == 2) {
+            const uint32_t u0 = p[t] & 0x03030303u;
+            const uint32_t u1 = (p[t] >> 2) & 0x03030303u;
+            const uint32_t u2 = (p[t] >> 4) & 0x03030303u;
+            const uint32_t u3 = (p[t] >> 6) & 0x03030303u;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const u32x4 a = act[act_index<BITS>(m, t, chunk, chunks_per_row)];
+                int r = raw[m];
+                r = dot4_i8(a.x, u0, r);
+                r = dot4_i8(a.y, u1, r);
+                r = dot4_i8(a.z, u2, r);
+                r = dot4_i8(a.w, u3, r);
+                raw[m] = r;
+            }
+        } else {
+            uint32_t u[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) u[j] = (p[t] >> j) & 0x01010101u;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const u32x4 a0 = act[act_index<BITS>(m, 2 * t, chunk, chunks_per_row)];
+                const u32x4 a1 = act[act_index<BITS>(m, 2 * t + 1, chunk, chunks_per_row)];
+                int r = raw[m];
+                r = dot4_i8(a0.x, u[0], r);
+                r = dot4_i8(a0.y, u[1], r);
+                r = dot4_i8(a0.z, u[2], r);
+                r = dot4_i8(a0.w, u[3], r);
+                r = dot4_i8(a1.x, u[4], r);
+                r = dot4_i8(a1.y, u[5], r);
+                r = dot4_i8(a1.z, u[6], r);
+                r = dot4_i8(a1.w, u[7], r);
+                raw[m] = r;
+            }
+        }
+    }
+}
+
+// Exact signed dot product of the chunk from the raw code dot and the chunk's
+// activation sum.
+template <int BITS>
+BONSAI_HD int chunk_dot_signed(int raw, int asum) {
+    return BITS == 2 ? raw - 2 * asum : 2 * raw - asum;
+}
+
+}  // namespace bonsai
+#endif  // BONSAI_GEMV_CORE_H

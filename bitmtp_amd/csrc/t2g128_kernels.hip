@@ -1,0 +1,36 @@
+// libbonsai_t2.so: C ABI of the T2-g128 (ternary, 2-bit codes) W2A8 GEMV for
+// gfx950.  Entry points are declared in include/bonsai_gemv.h; the drop-in one
+// replaces src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:123-148.
+#include "packed_gemv.hip.h"
+
+#include "../../include/bonsai_gemv.h"
+
+using namespace bonsai;
+
+extern "C" {
+
+int t2g128_init(void) { return init_device<2>(); }
+
+void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes) {
+    Tuning &t = lib_state<2>().tuning;
+    t.lanes_per_row = lanes_per_row;
+    t.waves_per_wg = waves_per_wg;
+    t.passes = passes;
+}
+
+int t2g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
+                   int M, int N, int K, int out_kind, int scale_kind, void *stream) {
+    return launch_gemv<2>(A, B, out, s, ws, M, N, K, out_kind, scale_kind,
+                          static_cast<hipStream_t>(stream));
+}
+
+void t2g128_int8xint2_linear(int8_t *A, int8_t *B, void *C, float *s, void *ws, int M, int N,
+                             int K, void *stream) {
+    const int rc = launch_gemv<2>(A, reinterpret_cast<const uint8_t *>(B), C, s, ws, M, N, K,
+                                  BONSAI_OUT_BF16, BONSAI_SCALE_BF16,
+                                  static_cast<hipStream_t>(stream));
+    if (rc != 0)
+        fprintf(stderr, "[t2g128] unsupported shape M=%d N=%d K=%d (status %d)\n", M, N, K, rc);
+}
+
+}  // extern "C"

@@ -1,0 +1,300 @@
+"""Packed low-bit GEMV operators for MI355X, mirroring the reference's operator
+boundary (src/bonsai_sft/gpu/model.py:66-268): the same function names, argument
+meaning, output shape/dtype and error behaviour, bound with ctypes to the gfx950
+libraries built by ``bitmtp_amd.build``.
+
+There is no CPU or PyTorch fallback: if a library is missing the loaders raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Tuple
+
+import torch
+
+from .contracts import require_kernel_shape
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+OUT_BF16, OUT_F32, OUT_G32 = 0, 1, 2
+SCALE_BF16, SCALE_F16 = 0, 1
+_X_KIND = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+_t2_lib = None
+_q1_lib = None
+_actq_lib = None
+
+_GEMV_ARGTYPES = [
+    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+    ctypes.c_void_p, ctypes.c_void_p,
+    ctypes.c_int, ctypes.c_int, ctypes.c_int,
+    ctypes.c_void_p,
+]
+_GEMV_EX_ARGTYPES = [
+    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+    ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+]
+
+
+def _open(relpath: str) -> ctypes.CDLL:
+    so = os.path.join(_HERE, relpath)
+    if not os.path.exists(so):
+        raise RuntimeError(
+            f"{so} is missing: build the gfx950 libraries with `python -m bitmtp_amd.build` "
+            "(there is no fallback implementation)")
+    return ctypes.CDLL(so)
+
+
+def t2_lib_path() -> str:
+    return os.path.join(_HERE, "t2g128_kernels", "libbonsai_t2.so")
+
+
+def q1_lib_path() -> str:
+    return os.path.join(_HERE, "q1g128_kernels", "libbonsai_q1.so")
+
+
+def actq_lib_path() -> str:
+    return os.path.join(_HERE, "act_quant", "libbonsai_actq.so")
+
+
+def load_t2_kernel() -> None:
+    """Load the T2-g128 INT8 x packed-INT2 library (reference: model.py:206-219)."""
+    global _t2_lib
+    lib = _open(os.path.join("t2g128_kernels", "libbonsai_t2.so"))
+    lib.t2g128_int8xint2_linear.argtypes = _GEMV_ARGTYPES
+    lib.t2g128_int8xint2_linear.restype = None
+    lib.t2g128_gemv_ex.argtypes = _GEMV_EX_ARGTYPES
+    lib.t2g128_gemv_ex.restype = ctypes.c_int
+    lib.t2g128_init.argtypes = []
+    lib.t2g128_init.restype = ctypes.c_int
+    lib.t2g128_set_tuning.argtypes = [ctypes.c_int] * 3
+    lib.t2g128_set_tuning.restype = None
+    _t2_lib = lib
+
+
+def load_q1_kernel() -> None:
+    """Load the Q1-g128 INT8 x packed-INT1 library (reference: model.py:70-93)."""
+    global _q1_lib
+    lib = _open(os.path.join("q1g128_kernels", "libbonsai_q1.so"))
+    lib.q1g128_int8xint1_linear.argtypes = _GEMV_ARGTYPES
+    lib.q1g128_int8xint1_linear.restype = None
+    lib.q1g128_w1a16_linear.argtypes = [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+    ]
+    lib.q1g128_w1a16_linear.restype = None
+    lib.q1g128_gemv_ex.argtypes = _GEMV_EX_ARGTYPES
+    lib.q1g128_gemv_ex.restype = ctypes.c_int
+    lib.q1g128_init.argtypes = []
+    lib.q1g128_init.restype = ctypes.c_int
+    lib.q1g128_set_tuning.argtypes = [ctypes.c_int] * 3
+    lib.q1g128_set_tuning.restype = None
+    _q1_lib = lib
+
+
+def load_actq_kernel() -> None:
+    global _actq_lib
+    lib = _open(os.path.join("act_quant", "libbonsai_actq.so"))
+    lib.bonsai_act_quant_int8.argtypes = [
+        ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+        ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+    ]
+    lib.bonsai_act_quant_int8.restype = ctypes.c_int
+    _actq_lib = lib
+
+
+def t2_lib() -> ctypes.CDLL:
+    if _t2_lib is None:
+        load_t2_kernel()
+    return _t2_lib
+
+
+def q1_lib() -> ctypes.CDLL:
+    if _q1_lib is None:
+        load_q1_kernel()
+    return _q1_lib
+
+
+def actq_lib() -> ctypes.CDLL:
+    if _actq_lib is None:
+        load_actq_kernel()
+    return _actq_lib
+
+
+def init_kernels() -> None:
+    """One-time per-device set-up of both GEMV libraries; call before graph capture."""
+    if t2_lib().t2g128_init() != 0 or q1_lib().q1g128_init() != 0:
+        raise RuntimeError("bonsai GEMV kernel initialisation failed on the current device")
+
+
+def _validate_packed_inputs(a, b, s, ws, *, kind, bits, activation_dtype,
+                            scale_dtypes=(torch.bfloat16,)):
+    """Tensor metadata checks before a native call, in the reference's order and
+    with its messages (model.py:96-115)."""
+    if a.dim() not in (2, 3) or b.dim() != 2:
+        raise ValueError(f"{kind}: expected rank-2/3 activation and rank-2 weight")
+    m = a.numel() // a.shape[-1] if a.shape[-1] else 0
+    n, k = b.shape[0], b.shape[1] * (8 // bits)
+    require_kernel_shape(kind, m, n, k)
+    if a.shape[-1] != k:
+        raise RuntimeError(f"{kind}: activation width mismatch: {a.shape[-1]} != {k}")
+    if tuple(ws.shape) != (n, k // 128):
+        raise RuntimeError(f"{kind}: invalid weight scale shape {tuple(ws.shape)}")
+    if a.dtype != activation_dtype or b.dtype != torch.int8 or ws.dtype not in scale_dtypes:
+        raise RuntimeError(f"{kind}: invalid activation, packed-weight, or scale dtype")
+    tensors = (a, b, ws) if s is None else (a, b, s, ws)
+    if s is not None and (s.dtype != torch.float32 or s.shape[-1:] != (1,) or s.numel() != m):
+        raise RuntimeError(f"{kind}: activation scales must be float32 with one value per row")
+    if not all(t.is_cuda and t.is_contiguous() for t in tensors):
+        raise RuntimeError(f"{kind}: inputs and scales must be contiguous CUDA tensors")
+    if not all(t.device == a.device for t in tensors):
+        raise RuntimeError(f"{kind}: inputs and scales must share one CUDA device")
+
+
+def _out_shape(a: torch.Tensor, n: int, kind: str) -> Tuple[int, Tuple[int, ...]]:
+    if a.dim() == 2:
+        return a.shape[0], (a.shape[0], n)
+    if a.dim() == 3:
+        bsz, slen, _ = a.shape
+        return bsz * slen, (bsz, slen, n)
+    raise ValueError(f"{kind} wrapper: bad input shape {a.shape}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(None if t is None else t.data_ptr())
+
+
+def _stream(device: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def t2g128_int8xint2_linear(a_int8: torch.Tensor, b_packed: torch.Tensor, s: torch.Tensor,
+                            ws: torch.Tensor) -> torch.Tensor:
+    """``[..., K] int8 x [N, K/4] packed ternary -> [..., N] bf16`` on the current
+    stream (reference: model.py:222-256)."""
+    _validate_packed_inputs(a_int8, b_packed, s, ws, kind="t2g128", bits=2,
+                            activation_dtype=torch.int8)
+    n, k = b_packed.shape[0], b_packed.shape[1] * 4
+    m, out_shape = _out_shape(a_int8, n, "t2g128")
+    lib = t2_lib()
+    out = torch.empty(*out_shape, dtype=torch.bfloat16, device=a_int8.device)
+    with torch.cuda.device(a_int8.device):
+        lib.t2g128_int8xint2_linear(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws),
+                                    m, n, k, _stream(a_int8.device))
+    return out
+
+
+def q1g128_int8xint1_linear(a_int8: torch.Tensor, b_packed: torch.Tensor, s: torch.Tensor,
+                            ws: torch.Tensor) -> torch.Tensor:
+    """``[..., K] int8 x [N, K/8] packed signs -> [..., N] bf16`` (reference:
+    model.py:118-153)."""
+    _validate_packed_inputs(a_int8, b_packed, s, ws, kind="q1", bits=1,
+                            activation_dtype=torch.int8)
+    n, k = b_packed.shape[0], b_packed.shape[1] * 8
+    m, out_shape = _out_shape(a_int8, n, "q1g128")
+    lib = q1_lib()
+    out = torch.empty(*out_shape, dtype=torch.bfloat16, device=a_int8.device)
+    with torch.cuda.device(a_int8.device):
+        lib.q1g128_int8xint1_linear(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws),
+                                    m, n, k, _stream(a_int8.device))
+    return out
+
+
+def q1g128_w1a16_linear(a_bf16: torch.Tensor, b_packed: torch.Tensor,
+                        ws: torch.Tensor) -> torch.Tensor:
+    """1-bit weights x bf16 activations, fp32 accumulation (reference: model.py:159-197).
+    The output is a fresh tensor from the caching allocator, which graph capture
+    tracks like any other allocation."""
+    if a_bf16.dim() != 2:
+        raise ValueError("w1a16 requires a rank-2 activation")
+    _validate_packed_inputs(a_bf16, b_packed, None, ws, kind="w1a16", bits=1,
+                            activation_dtype=torch.bfloat16)
+    m, n, k = a_bf16.shape[0], b_packed.shape[0], b_packed.shape[1] * 8
+    lib = q1_lib()
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=a_bf16.device)
+    with torch.cuda.device(a_bf16.device):
+        lib.q1g128_w1a16_linear(_ptr(a_bf16), _ptr(b_packed), _ptr(out), _ptr(ws), m, n, k,
+                                _stream(a_bf16.device))
+    return out
+
+
+def packed_int8_linear(a_int8, b_packed, s, ws):
+    """Dispatch by packed width: Q1 has K/8 bytes per row, T2 has K/4
+    (reference: model.py:259-268)."""
+    K = a_int8.shape[-1]
+    if b_packed.shape[-1] * 8 == K:
+        return q1g128_int8xint1_linear(a_int8, b_packed, s, ws)
+    if b_packed.shape[-1] * 4 == K:
+        return t2g128_int8xint2_linear(a_int8, b_packed, s, ws)
+    raise ValueError(
+        f"unknown packed weight layout A.K={K}, B.shape={tuple(b_packed.shape)}"
+    )
+
+
+def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[torch.Tensor],
+                   ws: Optional[torch.Tensor], *, bits: int, out_kind: int = OUT_BF16) -> torch.Tensor:
+    """The same kernels with a selectable result: bf16 ``[M,N]``, the fp32 value
+    before the bf16 rounding, or the exact int32 group sums ``[M,N,K/128]``.
+    ``ws`` may be bf16 or fp16.  Rank-2 activations only."""
+    if bits not in (1, 2):
+        raise ValueError("bits must be 1 (Q1) or 2 (T2)")
+    kind = "t2g128" if bits == 2 else "q1"
+    if out_kind == OUT_G32:
+        if a_int8.dim() != 2 or b_packed.dim() != 2:
+            raise ValueError(f"{kind}: expected rank-2 activation and rank-2 weight")
+        n, k = b_packed.shape[0], b_packed.shape[1] * (8 // bits)
+        require_kernel_shape(kind, a_int8.shape[0], n, k)
+        if a_int8.shape[-1] != k or a_int8.dtype != torch.int8 or b_packed.dtype != torch.int8:
+            raise RuntimeError(f"{kind}: invalid activation or packed-weight tensor")
+        if not (a_int8.is_cuda and b_packed.is_cuda and a_int8.is_contiguous()
+                and b_packed.is_contiguous()):
+            raise RuntimeError(f"{kind}: inputs must be contiguous CUDA tensors")
+    else:
+        if a_int8.dim() != 2:
+            raise ValueError(f"{kind}: expected rank-2 activation")
+        _validate_packed_inputs(a_int8, b_packed, s, ws, kind=kind, bits=bits,
+                                activation_dtype=torch.int8,
+                                scale_dtypes=(torch.bfloat16, torch.float16))
+    m, n, k = a_int8.shape[0], b_packed.shape[0], b_packed.shape[1] * (8 // bits)
+    dev = a_int8.device
+    if out_kind == OUT_BF16:
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    elif out_kind == OUT_F32:
+        out = torch.empty(m, n, dtype=torch.float32, device=dev)
+    elif out_kind == OUT_G32:
+        out = torch.empty(m, n, k // 128, dtype=torch.int32, device=dev)
+    else:
+        raise ValueError("bad out_kind")
+    scale_kind = SCALE_F16 if (ws is not None and ws.dtype == torch.float16) else SCALE_BF16
+    fn = t2_lib().t2g128_gemv_ex if bits == 2 else q1_lib().q1g128_gemv_ex
+    with torch.cuda.device(dev):
+        rc = fn(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws), m, n, k, out_kind,
+                scale_kind, _stream(dev))
+    if rc != 0:
+        raise RuntimeError(f"{kind}: native launch failed with status {rc} (M={m}, N={n}, K={k})")
+    return out
+
+
+def quant_input(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-token absmax INT8 quantisation on the GPU: returns ``(q int8 [..., K],
+    s fp32 [..., 1])`` with ``s = 127 / clamp_min(absmax, 1e-5)`` (reference:
+    model.py:632-636)."""
+    if x.dtype not in _X_KIND:
+        raise RuntimeError("quant_input: activation must be bfloat16, float16 or float32")
+    if not (x.is_cuda and x.is_contiguous()) or x.dim() < 1:
+        raise RuntimeError("quant_input: activation must be a contiguous CUDA tensor")
+    k = x.shape[-1]
+    if k == 0 or k % 8 != 0:
+        raise RuntimeError("quant_input: last dimension must be a positive multiple of 8")
+    m = x.numel() // k
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty(*x.shape[:-1], 1, dtype=torch.float32, device=x.device)
+    if m == 0:
+        return q, s
+    with torch.cuda.device(x.device):
+        rc = actq_lib().bonsai_act_quant_int8(_ptr(x), _X_KIND[x.dtype], _ptr(q), _ptr(s), m, k,
+                                              _stream(x.device))
+    if rc != 0:
+        raise RuntimeError(f"quant_input: native launch failed with status {rc}")
+    return q, s

@@ -1,0 +1,117 @@
+/*
+ * C ABI of the MI355X (gfx950) packed low-bit GEMV libraries.
+ *
+ *   libbonsai_t2.so      T2-g128 ternary weights (2-bit codes), int8 activations
+ *   libbonsai_q1.so      Q1-g128 sign weights   (1 bit),       int8 activations
+ *   libbonsai_actq.so    per-token absmax INT8 activation quantisation
+ *
+ * Plain pointers and sizes only; every pointer is DEVICE memory unless stated.
+ * Nothing here synchronises the host, allocates, frees or retains a pointer;
+ * all work is enqueued on `stream` (a hipStream_t passed as void*), so every
+ * entry point may be called while that stream is being captured into a graph.
+ *
+ * Operand layout (identical to the reference kernels,
+ * src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:3-8 and
+ * src/bonsai_sft/gpu/q1g128_kernels/q1g128_kernels.h:14-24):
+ *   A   int8  [M, K]        row-major, per-token quantised activations
+ *   B   uint8 [N, K/4]      T2: weight k of row n = ((B[n][k/4] >> 2(k%4)) & 3) - 2
+ *       uint8 [N, K/8]      Q1: weight k of row n = 2*((B[n][k/8] >> (k%8)) & 1) - 1
+ *   ws  16-bit [N, K/128]   one scale per row and 128-wide K group (bf16; the
+ *                           *_f16s entry points read IEEE fp16 instead)
+ *   s   fp32  [M]           activation MULTIPLIER 127/absmax (the result is divided by it)
+ *   C   bf16  [M, N]        C[m][n] = bf16( (sum_g fp32(G[m][n][g]) * ws[n][g]) / s[m] )
+ *   G   int32 [M, N, K/128] exact group sums G[m][n][g] = sum_{k in g} A[m][k] * w[n][k]
+ *
+ * Preconditions: M >= 1, N >= 1, K >= 128 and K % 128 == 0, B rows 16-byte
+ * aligned (true for every K % 128 == 0 when B itself is 16-byte aligned), A
+ * 16-byte aligned.  Any M is accepted: widths above 8 are processed as several
+ * token tiles inside one launch.
+ */
+#ifndef BONSAI_GEMV_H
+#define BONSAI_GEMV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes of the int-returning entry points. */
+#define BONSAI_OK 0
+#define BONSAI_ERR_ARG 1    /* null pointer, M/N/K out of range, K % 128 != 0 */
+#define BONSAI_ERR_LAUNCH 2 /* hipLaunchKernel / attribute call failed */
+
+/* ---- drop-in entry points ------------------------------------------------ */
+
+/* Replaces `t2g128_int8xint2_linear`
+ * (src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:123-148), bound by ctypes
+ * at src/bonsai_sft/gpu/model.py:206-219 with argtypes 5 x void*, 3 x int, void*.
+ * Like the reference it returns nothing: on a violated precondition it prints
+ * one line to stderr and leaves C untouched.  Unlike the reference it has no
+ * table of registered (M,N,K): every shape meeting the preconditions runs. */
+void t2g128_int8xint2_linear(int8_t *A, int8_t *B, void *C /* bf16 */, float *s,
+                             void *ws /* bf16 */, int M, int N, int K, void *stream);
+
+/* Replaces `q1g128_int8xint1_linear`
+ * (src/bonsai_sft/gpu/q1g128_kernels/q1g128_kernels_block8.cu:118-241), bound at
+ * src/bonsai_sft/gpu/model.py:70-93.  Same contract as above with 1-bit weights. */
+void q1g128_int8xint1_linear(int8_t *A, int8_t *B, void *C /* bf16 */, float *s,
+                             void *ws /* bf16 */, int M, int N, int K, void *stream);
+
+/* Replaces `q1g128_w1a16_linear`
+ * (src/bonsai_sft/gpu/q1g128_kernels/q1g128_kernels_block8.cu:93-112): 1-bit
+ * weights times bf16 activations with fp32 accumulation and no activation
+ * scale, C[m][n] = bf16( sum_g ws[n][g] * sum_{k in g} fp32(A[m][k]) * w[n][k] ).
+ * Exported because the reference loader binds it together with the symbol
+ * above (model.py:86-91). */
+void q1g128_w1a16_linear(const void *A /* bf16 [M,K] */, const int8_t *B, void *C /* bf16 */,
+                         const void *ws /* bf16 */, int M, int N, int K, void *stream);
+
+/* ---- checked variants of the same kernels -------------------------------- */
+/* Same kernels as the drop-in entry points, selected by `out_kind`, with a
+ * status code instead of a message.  They exist so that tests and callers can
+ * read the exact int32 group sums and the fp32 value before the bf16 rounding
+ * (the reference has no counterpart; its CUDA kernels keep both in registers,
+ * t2g128_kernels.cu:74-90). */
+#define BONSAI_OUT_BF16 0 /* out = bf16 [M,N]                                  */
+#define BONSAI_OUT_F32 1  /* out = fp32 [M,N], value before rounding to bf16  */
+#define BONSAI_OUT_G32 2  /* out = int32 [M,N,K/128]; s and ws are not read    */
+
+#define BONSAI_SCALE_BF16 0
+#define BONSAI_SCALE_F16 1
+
+int t2g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
+                   int M, int N, int K, int out_kind, int scale_kind, void *stream);
+int q1g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
+                   int M, int N, int K, int out_kind, int scale_kind, void *stream);
+
+/* One-time set-up for the current device (raises the kernels' dynamic-LDS
+ * limit).  Called implicitly by the first launch; call it explicitly before
+ * capturing a graph if the first launch would otherwise happen under capture.
+ * No reference counterpart (the CUDA kernels use no shared memory). */
+int t2g128_init(void);
+int q1g128_init(void);
+
+/* Launch-geometry override for tuning experiments: lanes per weight row
+ * (4..64, power of two), waves per workgroup (1..16) and row passes per wave
+ * (>= 1).  Zero restores the built-in heuristic for that field.  Process-wide,
+ * not thread-safe; no reference counterpart. */
+void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
+void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
+
+/* ---- activation quantisation (libbonsai_actq.so) ------------------------- */
+/* Per-token symmetric INT8 quantisation, the native form of `quant_input`
+ * (src/bonsai_sft/gpu/model.py:632-636, identical copy at :571-575):
+ *   s[m] = 127 / max(max_k |x[m][k]|, 1e-5)          (fp32)
+ *   q[m][k] = clamp(round_half_even(fp32(x[m][k]) * s[m]), -128, 127)
+ * x_kind selects the element type of x. */
+#define BONSAI_X_BF16 0
+#define BONSAI_X_F16 1
+#define BONSAI_X_F32 2
+int bonsai_act_quant_int8(const void *x, int x_kind, int8_t *q, float *s, int M, int K,
+                          void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BONSAI_GEMV_H */
