@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed T2-g128 GEMV hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): all seven linear projections of one
+Qwen3-1.7B-shaped decoder layer in T2-g128 -- q/o 2048x2048, k/v 1024x2048,
+gate/up 6144x2048, down 2048x6144 -- at widths 1, 4 and 8, through the drop-in
+C entry point ``t2g128_int8xint2_linear``.  One STEP is that set once: 3 widths x
+7 projections = 21 launches.  Every launch reads a different layer of a pool of
+distinct random layers larger than the 256 MB Infinity Cache, so the weights come
+from HBM, and the steps are replayed from one HIP graph so that the Python launch
+cost is outside the measurement, as in the reference's graph-replayed decode.
+
+Prints ONE JSON line (see README / DESIGN.md for the fields).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+WIDTHS = (1, 4, 8)
+# name, N, K  (Qwen3-1.7B: hidden 2048, 16 q / 8 kv heads x 128, ffn 6144)
+PROJECTIONS = (
+    ("q_proj", 2048, 2048), ("k_proj", 1024, 2048), ("v_proj", 1024, 2048),
+    ("o_proj", 2048, 2048), ("gate_proj", 6144, 2048), ("up_proj", 6144, 2048),
+    ("down_proj", 2048, 6144),
+)
+
+
+def t2_bytes(n: int, k: int) -> int:
+    """Algorithmic bytes of one T2 GEMV: packed weights + group scales."""
+    return n * k // 4 + n * (k // 128) * 2
+
+
+LAYER_BYTES = sum(t2_bytes(n, k) for _, n, k in PROJECTIONS)  # 13,369,344
+
+
+def make_pool(torch, n_layers: int, seed: int, dev):
+    """Seeded i.i.d. ternary weights (p = 1/3 each, codes 1..3 packed four per byte)
+    and log-normal(-4, 0.5) group scales rounded to bf16."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    shifts = torch.tensor([1, 4, 16, 64], device=dev, dtype=torch.int32)
+    pool = []
+    for _ in range(n_layers):
+        layer = []
+        for _, n, k in PROJECTIONS:
+            codes = torch.randint(1, 4, (n, k // 4, 4), generator=gen, device=dev, dtype=torch.int32)
+            packed = (codes * shifts).sum(-1).to(torch.uint8).view(torch.int8).contiguous()
+            scales = torch.exp(torch.randn(n, k // 128, generator=gen, device=dev) * 0.5 - 4.0)
+            layer.append((packed, scales.to(torch.bfloat16).contiguous()))
+        pool.append(layer)
+    return pool
+
+
+def make_activations(torch, ops, seed: int, dev):
+    """fp16 N(0,1) activations per width and K, quantised per token on the GPU."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed + 1)
+    acts = {}
+    for m in WIDTHS:
+        for k in sorted({k for _, _, k in PROJECTIONS}):
+            x = torch.randn(m, k, generator=gen, device=dev).to(torch.float16)
+            q, s = ops.quant_input(x)
+            acts[(m, k)] = (q, s)
+    return acts
+
+
+class Runner:
+    def __init__(self, torch, ops_mod, pool, acts, dev):
+        self.torch = torch
+        self.pool = pool
+        self.acts = acts
+        self.fn = ops_mod.t2_lib().t2g128_int8xint2_linear
+        self.outs = {(m, i): torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+                     for m in WIDTHS for i, (_, n, _) in enumerate(PROJECTIONS)}
+        self.cursor = 0  # next pool layer
+
+    def launch_layer(self, m: int, stream_ptr):
+        layer = self.pool[self.cursor % len(self.pool)]
+        self.cursor += 1
+        for i, (_, n, k) in enumerate(PROJECTIONS):
+            q, s = self.acts[(m, k)]
+            packed, scales = layer[i]
+            self.fn(q.data_ptr(), packed.data_ptr(), self.outs[(m, i)].data_ptr(), s.data_ptr(),
+                    scales.data_ptr(), m, n, k, stream_ptr)
+
+    def step(self, widths, stream_ptr):
+        for m in widths:
+            self.launch_layer(m, stream_ptr)
+
+    def capture(self, n_steps: int, widths):
+        torch = self.torch
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for _ in range(n_steps):
+                self.step(widths, sp)
+        return g
+
+    def time_graph(self, g) -> float:
+        torch = self.torch
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3  # seconds
+
+
+def cpu_baseline(budget_s: float):
+    """Times the C oracle (OpenMP over output rows) on one layer at widths 1, 4, 8 --
+    the same 21 GEMVs as one step -- repeating it until about `budget_s` seconds."""
+    import numpy as np
+    from oracle import oracle as O
+    O.build()
+    problems = []
+    for m in WIDTHS:
+        for _, n, k in PROJECTIONS:
+            problems.append(O.synth_problem(1, m, n, k, 2))
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    reps, t_used = 0, 0.0
+    while t_used < budget_s and reps < 1000:
+        t0 = time.perf_counter()
+        for p in problems:
+            O.c_gemv(p["A"], p["B"], p["s"], p["ws"], 2)
+        t_used += time.perf_counter() - t0
+        reps += 1
+    total_bytes = reps * len(WIDTHS) * LAYER_BYTES
+    return {
+        "value": round(total_bytes / t_used / 1e9, 3), "unit": "GB/s", "cores": threads,
+        "kind": "port",
+        "sample": f"{reps} x (one 1.7B-shaped layer, 7 T2 projections at widths 1,4,8) in "
+                  f"{t_used:.1f} s with the C oracle, OpenMP over rows",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=192)
+    ap.add_argument("--warmup", type=int, default=24)
+    ap.add_argument("--layers", type=int, default=48, help="distinct layers in the weight pool")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 256 MiB device copy (for scaling rocprofv3 PMC byte counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (--gpus must be 1)",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    import bitmtp_amd as ops
+    from bitmtp_amd import ops as ops_mod
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    ops.init_kernels()
+
+    pool = make_pool(torch, args.layers, seed=1, dev=dev)
+    acts = make_activations(torch, ops, seed=1, dev=dev)
+    run = Runner(torch, ops_mod, pool, acts, dev)
+
+    # warm-up: eager steps (loads code objects), then one untimed replay of the timed graph
+    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(max(args.warmup, 1)):
+        run.step(WIDTHS, sp)
+    torch.cuda.synchronize()
+
+    run.cursor = 0
+    graph = run.capture(args.steps, WIDTHS)
+    graph.replay()
+    torch.cuda.synchronize()
+    elapsed = min(run.time_graph(graph) for _ in range(3))
+
+    step_bytes = len(WIDTHS) * LAYER_BYTES
+    gbps = step_bytes * args.steps / elapsed / 1e9
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # per-width: the same stream with one width only (7 launches per step)
+    per_width = {}
+    for m in WIDTHS:
+        run.cursor = 0
+        g = run.capture(args.steps, (m,))
+        g.replay()
+        torch.cuda.synchronize()
+        t = min(run.time_graph(g) for _ in range(3))
+        launches = args.steps * len(PROJECTIONS)
+        per_width[m] = {
+            "gbps": round(LAYER_BYTES * args.steps / t / 1e9, 1),
+            "pct_hbm_peak": round(LAYER_BYTES * args.steps / t / 1e9 / HBM_PEAK_GBPS * 100, 2),
+            "us_per_layer": round(t / args.steps * 1e6, 3),
+            "us_per_launch": round(t / launches * 1e6, 3),
+        }
+        del g
+
+    # roofline of the dominant kernel: the width whose launches take the most time
+    dom = max(WIDTHS, key=lambda m: per_width[m]["us_per_launch"])
+    bytes_per_launch = LAYER_BYTES / len(PROJECTIONS)
+    achieved = bytes_per_launch / (per_width[dom]["us_per_launch"] * 1e-6) / 1e9
+    roofline = {
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "kernel": f"gemv_dot4_kernel<BITS=2, MT={dom}, OUT=bf16> (width {dom})",
+        "bytes_per_launch": round(bytes_per_launch),
+        "us_per_launch": per_width[dom]["us_per_launch"],
+    }
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+
+    cpu = cpu_baseline(args.cpu_seconds) if args.cpu_seconds > 0 else None
+
+    line = {
+        "metric": "t2g128_packed_gemv_hbm_throughput", "value": round(gbps, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: 7 T2-g128 projections of one Qwen3-1.7B-shaped layer at "
+                        "widths 1,4,8 (21 launches/step), HBM-cold over a pool of distinct layers",
+            "pool_layers": args.layers, "pool_bytes": args.layers * LAYER_BYTES,
+            "bytes_per_step": step_bytes, "launches_per_step": len(WIDTHS) * len(PROJECTIONS),
+            "pct_hbm_peak": round(gbps / HBM_PEAK_GBPS * 100, 2),
+            "per_width": {str(m): per_width[m] for m in WIDTHS},
+            "timing": "one HIP graph of all steps, HIP events on the launch stream, best of 3 replays",
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

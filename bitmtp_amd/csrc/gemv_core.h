@@ -36,6 +36,15 @@
 #define BONSAI_HD inline
 #endif
 
+// Scheduling fence for the device compiler: nothing is moved across it.  Used to
+// bound how many LDS reads are hoisted ahead of the arithmetic that consumes
+// them (each costs four registers).
+#if defined(__HIP_DEVICE_COMPILE__)
+#define BONSAI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define BONSAI_SCHED_FENCE() ((void)0)
+#endif
+
 namespace bonsai {
 
 struct alignas(16) u32x4 {
@@ -88,48 +97,66 @@ BONSAI_HD u32x4 transpose4x4_bytes(uint32_t i0, uint32_t i1, uint32_t i2, uint32
 
 BONSAI_HD int sum4_i8(uint32_t a) { return dot4_i8(a, 0x01010101u, 0); }
 
-// Index of activation unit `unit` of chunk `chunk` for tile token `m` in the
-// staged array (16-byte elements).  Units are the slow index so that the lanes
-// of a wave, which hold consecutive chunks, read consecutive 16-byte words.
-template <int BITS>
-BONSAI_HD int act_index(int m, int unit, int chunk, int chunks_per_row) {
-    return (m * Fmt<BITS>::kUnits + unit) * chunks_per_row + chunk;
+// Staged-activation layout (LDS on the GPU).  Everything one weight chunk needs
+// lives in one BLOCK of `block_words<BITS, MT>()` 16-byte words:
+//     words [m*kUnits + unit]      permuted activation unit `unit` of tile token m
+//     words [MT*kUnits ...]        MT int32 chunk activation sums (asum), then padding
+// so that a lane addresses all of it with one base register and immediate
+// offsets.  The block size is odd: lanes holding consecutive chunks then hit
+// distinct 16-byte bank groups, whatever MT is.
+template <int BITS, int MT>
+BONSAI_HD constexpr int block_words() {
+    return ((MT * Fmt<BITS>::kUnits + (MT * 4 + 15) / 16) | 1);
 }
 
-// Stage one chunk of one token: `src` points at the chunk's kChunkWeights
-// natural-order int8 activations (16-byte aligned); writes kUnits permuted
-// units into act[] and returns the sum of the chunk's activations.
-template <int BITS>
-BONSAI_HD int stage_chunk(const u32x4 *src, u32x4 *act, int m, int chunk, int chunks_per_row) {
-    int sum = 0;
+template <int BITS, int MT>
+BONSAI_HD int act_index(int m, int unit, int chunk) {
+    return chunk * block_words<BITS, MT>() + m * Fmt<BITS>::kUnits + unit;
+}
+
+// Index (in int32 units) of the activation sum of token m for `chunk`.
+template <int BITS, int MT>
+BONSAI_HD int asum_index(int m, int chunk) {
+    return (chunk * block_words<BITS, MT>() + MT * Fmt<BITS>::kUnits) * 4 + m;
+}
+
+// Stage one quarter (`sub` = 0..3) of one chunk of one token.  `src` points at the
+// quarter's natural-order int8 activations (16 for T2, 32 for Q1; 16-byte
+// aligned).  Writes the permuted unit(s) into act[] and returns the sum of the
+// quarter's activations; the four quarter sums of a chunk add up to its asum.
+template <int BITS, int MT>
+BONSAI_HD int stage_quarter(const u32x4 *src, u32x4 *act, int m, int chunk, int sub) {
     if (BITS == 2) {
-        for (int t = 0; t < 4; ++t) {
-            u32x4 in = src[t];  // activations 16t .. 16t+15
-            sum += sum4_i8(in.x) + sum4_i8(in.y) + sum4_i8(in.z) + sum4_i8(in.w);
-            // unit t, dword j, byte b  <-  activation 16t + 4b + j
-            act[act_index<BITS>(m, t, chunk, chunks_per_row)] =
-                transpose4x4_bytes(in.x, in.y, in.z, in.w);
-        }
+        const u32x4 in = src[0];  // activations 16*sub .. 16*sub+15 of the chunk
+        // unit sub, dword j, byte b  <-  activation 16*sub + 4b + j
+        act[act_index<BITS, MT>(m, sub, chunk)] =
+            transpose4x4_bytes(in.x, in.y, in.z, in.w);
+        return sum4_i8(in.x) + sum4_i8(in.y) + sum4_i8(in.z) + sum4_i8(in.w);
     } else {
-        for (int t = 0; t < 4; ++t) {
-            u32x4 lo = src[2 * t], hi = src[2 * t + 1];  // activations 32t .. 32t+31
-            sum += sum4_i8(lo.x) + sum4_i8(lo.y) + sum4_i8(lo.z) + sum4_i8(lo.w);
-            sum += sum4_i8(hi.x) + sum4_i8(hi.y) + sum4_i8(hi.z) + sum4_i8(hi.w);
-            // unit 2t+h, dword d, byte b  <-  activation 32t + 8b + 4h + d
-            act[act_index<BITS>(m, 2 * t, chunk, chunks_per_row)] =
-                transpose4x4_bytes(lo.x, lo.z, hi.x, hi.z);
-            act[act_index<BITS>(m, 2 * t + 1, chunk, chunks_per_row)] =
-                transpose4x4_bytes(lo.y, lo.w, hi.y, hi.w);
-        }
+        const u32x4 lo = src[0], hi = src[1];  // activations 32*sub .. 32*sub+31
+        // unit 2*sub+h, dword d, byte b  <-  activation 32*sub + 8b + 4h + d
+        act[act_index<BITS, MT>(m, 2 * sub, chunk)] =
+            transpose4x4_bytes(lo.x, lo.z, hi.x, hi.z);
+        act[act_index<BITS, MT>(m, 2 * sub + 1, chunk)] =
+            transpose4x4_bytes(lo.y, lo.w, hi.y, hi.w);
+        return sum4_i8(lo.x) + sum4_i8(lo.y) + sum4_i8(lo.z) + sum4_i8(lo.w) +
+               sum4_i8(hi.x) + sum4_i8(hi.y) + sum4_i8(hi.z) + sum4_i8(hi.w);
     }
+}
+
+// Stage a whole chunk (the four quarters in turn); returns the chunk's asum.
+template <int BITS, int MT>
+BONSAI_HD int stage_chunk(const u32x4 *src, u32x4 *act, int m, int chunk) {
+    int sum = 0;
+    for (int sub = 0; sub < 4; ++sub)
+        sum += stage_quarter<BITS, MT>(src + sub * (Fmt<BITS>::kUnits / 4), act, m, chunk, sub);
     return sum;
 }
 
 // Raw dot products of one 16-byte weight chunk against MT staged tokens:
 // raw[m] += sum_k a[m][k] * code[k] (codes 0..3 for T2, bits 0..1 for Q1).
 template <int BITS, int MT>
-BONSAI_HD void chunk_dot_raw(const u32x4 w, const u32x4 *act, int chunk, int chunks_per_row,
-                             int raw[MT]) {
+BONSAI_HD void chunk_dot_raw(const u32x4 w, const u32x4 *act, int chunk, int raw[MT]) {
     const uint32_t p[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -140,7 +167,7 @@ BONSAI_HD void chunk_dot_raw(const u32x4 w, const u32x4 *act, int chunk, int chu
             const uint32_t u3 = (p[t] >> 6) & 0x03030303u;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                const u32x4 a = act[act_index<BITS>(m, t, chunk, chunks_per_row)];
+                const u32x4 a = act[act_index<BITS, MT>(m, t, chunk)];
                 int r = raw[m];
                 r = dot4_i8(a.x, u0, r);
                 r = dot4_i8(a.y, u1, r);
@@ -154,8 +181,8 @@ BONSAI_HD void chunk_dot_raw(const u32x4 w, const u32x4 *act, int chunk, int chu
             for (int j = 0; j < 8; ++j) u[j] = (p[t] >> j) & 0x01010101u;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                const u32x4 a0 = act[act_index<BITS>(m, 2 * t, chunk, chunks_per_row)];
-                const u32x4 a1 = act[act_index<BITS>(m, 2 * t + 1, chunk, chunks_per_row)];
+                const u32x4 a0 = act[act_index<BITS, MT>(m, 2 * t, chunk)];
+                const u32x4 a1 = act[act_index<BITS, MT>(m, 2 * t + 1, chunk)];
                 int r = raw[m];
                 r = dot4_i8(a0.x, u[0], r);
                 r = dot4_i8(a0.y, u[1], r);

@@ -31,9 +31,8 @@
 namespace bonsai {
 
 constexpr int kGroup = 128;
-constexpr int kMaxTile = 8;      // tokens per tile (template MT is 1..kMaxTile)
-constexpr int kBatch = 4;        // 16-byte weight loads in flight per lane and batch
-constexpr int kMaxThreads = 512; // workgroup size limit of the kernels
+constexpr int kMaxTile = 8;       // tokens per tile (template MT is 1..kMaxTile)
+constexpr int kMaxThreads = 512;  // workgroup size limit of the kernels
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_G32 = 2 };
 
@@ -44,8 +43,10 @@ struct GemvArgs {
     const float *s;
     const uint16_t *ws;
     int M, N, K;
-    int lpr_log2;  // log2(lanes per weight row)
-    int passes;    // row passes per wave
+    int lpr_log2;        // log2(lanes per weight row)
+    int passes;          // row passes per wave
+    int out_f32;         // 1: store the fp32 value, 0: round to bf16
+    uint32_t div_magic;  // floor(2^32 / (4*C)) + 1, for task -> token in the staging loop
 };
 
 template <bool SF16>
@@ -71,10 +72,10 @@ __device__ __forceinline__ int dpp_i32(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
 }
 
-constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
-constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
-constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8 lanes
-constexpr int kDppMirror = 0x140;     // lane i <-> 15-i inside each 16 lanes
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7-i inside each 8 lanes
+constexpr int kDppMirror = 0x140;      // lane i <-> 15-i inside each 16 lanes
 
 // Sum over the 2^lpr_log2 consecutive lanes that share a weight row; every lane
 // of the set ends up with the total.
@@ -88,12 +89,17 @@ __device__ __forceinline__ float row_lanes_sum(float v, int lpr_log2) {
     return v;
 }
 
+// U 16-byte weight chunks of one lane plus the raw 16-bit scales of their groups.
+template <int U>
 struct WeightBatch {
-    u32x4 w[kBatch];
-    float sc[kBatch];  // group scale, 0 for lanes past the end of the row
+    u32x4 w[U];
+    uint16_t sraw[U];
 };
 
-template <int BITS, int MT, int OUT, bool SF16>
+// BITS: 2 = T2, 1 = Q1.  MT: tokens in the tile.  U: 16-byte weight loads a lane
+// issues back to back (one batch).  G32: write the int32 group sums instead of
+// the scaled result.  SF16: group scales are fp16 instead of bf16.
+template <int BITS, int MT, int U, bool G32, bool SF16>
 __global__ void __launch_bounds__(kMaxThreads) gemv_dot4_kernel(const GemvArgs a) {
     using F = Fmt<BITS>;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -101,57 +107,86 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_dot4_kernel(const GemvArgs a
     const int K = a.K, N = a.N, M = a.M;
     const int C = K / F::kChunkWeights;  // 16-byte chunks per weight row
     const int ng = K / kGroup;
-    const size_t row_bytes = (size_t)C * 16;
 
-    u32x4 *act = reinterpret_cast<u32x4 *>(smem);                 // [MT][kUnits][C]
-    int *asum = reinterpret_cast<int *>(smem + (size_t)MT * K);   // [MT][C]
+    u32x4 *act = reinterpret_cast<u32x4 *>(smem);  // C blocks, see gemv_core.h
+    int *asum = reinterpret_cast<int *>(smem);
 
     const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int nwaves = blockDim.x >> 6;
+    const int nwaves = nthreads >> 6;
     const int lpr_log2 = a.lpr_log2;
     const int lpr = 1 << lpr_log2;
-    const int c = lane & (lpr - 1);        // position of the lane along K
-    const int r = lane >> lpr_log2;        // row of the lane inside the wave
-    const int rpw = 64 >> lpr_log2;        // rows per wave and pass
+    const int c = lane & (lpr - 1);  // position of the lane along K
+    const int r = lane >> lpr_log2;  // row of the lane inside the wave
+    const int rpw = 64 >> lpr_log2;  // rows per wave and pass
     const int IT = (C + lpr - 1) >> lpr_log2;
-    const int nb = (IT + kBatch - 1) / kBatch;
+    const int nb = (IT + U - 1) / U;
     const int m0 = blockIdx.y * MT;
+    const int row0 = ((int)blockIdx.x * a.passes * nwaves + wave) * rpw + r;
+    const int row_step = nwaves * rpw;  // rows between two passes of a wave
 
-    auto row_of = [&](int pass) {
-        return (((int)blockIdx.x * a.passes + pass) * nwaves + wave) * rpw + r;
-    };
-
-    auto load_batch = [&](WeightBatch &wb, int row, int it0) {
+    // All loads of a batch are unconditional (indices clamped into the row) and
+    // issued back to back; lanes past the end of a row are masked when used.
+    auto load_batch = [&](WeightBatch<U> &wb, int row, int it0) {
         const int row_c = row < N ? row : N - 1;
-        const u32x4 *wrow = reinterpret_cast<const u32x4 *>(a.B + (size_t)row_c * row_bytes);
+        const u32x4 *wrow = reinterpret_cast<const u32x4 *>(a.B) + (size_t)row_c * C;
         const uint16_t *srow = a.ws + (size_t)row_c * ng;
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            if (it0 + u >= IT) break;  // wave-uniform: the row has no such chunk column
+        for (int u = 0; u < U; ++u) {
             const int chunk = (it0 + u) * lpr + c;
             const int chunk_c = chunk < C ? chunk : C - 1;
             wb.w[u] = wrow[chunk_c];
-            if (OUT != OUT_G32) {
-                const float f = scale_to_f32<SF16>(srow[chunk_c >> F::kGroupShift]);
-                wb.sc[u] = (chunk < C && row < N) ? f : 0.0f;
-            }
+            if (!G32) wb.sraw[u] = srow[chunk_c >> F::kGroupShift];
         }
     };
 
-    // Weight loads for the first batch go out before the activations are
-    // staged, so that their HBM latency overlaps the staging.
-    WeightBatch cur, nxt;
-    load_batch(cur, row_of(0), 0);
-
-    for (int task = tid; task < MT * C; task += blockDim.x) {
-        const int m = task / C;
-        const int chunk = task - m * C;
+    // ---- prologue: first staging loads, then the first weight batch, so that the
+    // staging data (an L2 hit) is back before the weights (HBM) are.
+    const int ntasks = MT * C * 4;  // quarter chunks to stage
+    constexpr int kQ = F::kUnits / 4;  // 16-byte words per quarter
+    auto task_src = [&](int task, int &m, int &chunk, int &sub) {
+        m = (int)__umulhi((uint32_t)task, a.div_magic);  // task / (4*C)
+        const int rest = task - m * 4 * C;
+        chunk = rest >> 2;
+        sub = rest & 3;
         const int msrc = (m0 + m) < M ? (m0 + m) : M - 1;
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.A + (size_t)msrc * K) +
-                           (size_t)chunk * F::kUnits;
-        asum[m * C + chunk] = stage_chunk<BITS>(src, act, m, chunk, C);
+        return reinterpret_cast<const u32x4 *>(a.A + (size_t)msrc * K) +
+               ((size_t)chunk * 4 + sub) * kQ;
+    };
+    u32x4 first_q[kQ];
+    int fm = 0, fchunk = 0, fsub = 0;
+    const bool has_first = tid < ntasks;
+    if (has_first) {
+        const u32x4 *src = task_src(tid, fm, fchunk, fsub);
+#pragma unroll
+        for (int i = 0; i < kQ; ++i) first_q[i] = src[i];
+    }
+
+    WeightBatch<U> cur, nxt;
+    load_batch(cur, row0, 0);
+
+    float sdiv[MT];
+    if (!G32) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) sdiv[m] = a.s[(m0 + m) < M ? (m0 + m) : M - 1];
+    }
+
+    // ---- stage the token tile: permuted activations and per-chunk sums into LDS
+    if (has_first) {
+        int qs = stage_quarter<BITS, MT>(first_q, act, fm, fchunk, fsub);
+        qs += dpp_i32<kDppXor1>(qs);
+        qs += dpp_i32<kDppXor2>(qs);
+        if (fsub == 0) asum[asum_index<BITS, MT>(fm, fchunk)] = qs;
+    }
+    for (int task = tid + nthreads; task < ntasks; task += nthreads) {
+        int m, chunk, sub;
+        const u32x4 *src = task_src(task, m, chunk, sub);
+        int qs = stage_quarter<BITS, MT>(src, act, m, chunk, sub);
+        qs += dpp_i32<kDppXor1>(qs);
+        qs += dpp_i32<kDppXor2>(qs);
+        if (sub == 0) asum[asum_index<BITS, MT>(m, chunk)] = qs;
     }
     __syncthreads();
 
@@ -159,52 +194,47 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_dot4_kernel(const GemvArgs a
 #pragma unroll
     for (int m = 0; m < MT; ++m) accf[m] = 0.0f;
 
-    const int total = a.passes * nb;
-    int pass = 0, b = 0;
-    for (int i = 0; i < total; ++i) {
-        int npass = pass, nbt = b + 1;
-        if (nbt == nb) {
-            nbt = 0;
-            npass = pass + 1;
-        }
-        const bool more = i + 1 < total;
-        if (more) load_batch(nxt, row_of(npass), nbt * kBatch);
-
-        const int row = row_of(pass);
+    // One batch of one pass: unpack, dot, scale, and after the last batch of the
+    // pass reduce over the row's lanes and store.
+    auto compute_batch = [&](const WeightBatch<U> &wb, int pass, int b) {
+        const int row = row0 + pass * row_step;
+        const bool row_ok = row < N;
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            if (b * kBatch + u >= IT) break;  // wave-uniform
-            const int chunk = (b * kBatch + u) * lpr + c;
+        for (int u = 0; u < U; ++u) {
+            const int chunk = (b * U + u) * lpr + c;
+            const bool ok = row_ok && chunk < C;
             const int chunk_c = chunk < C ? chunk : C - 1;
             int raw[MT];
 #pragma unroll
             for (int m = 0; m < MT; ++m) raw[m] = 0;
-            chunk_dot_raw<BITS, MT>(cur.w[u], act, chunk_c, C, raw);
+            chunk_dot_raw<BITS, MT>(wb.w[u], act, chunk_c, raw);
+            float wsf = 0.0f;
+            if (!G32) wsf = scale_to_f32<SF16>(wb.sraw[u]);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-                int g = chunk_dot_signed<BITS>(raw[m], asum[m * C + chunk_c]);
-                if (OUT == OUT_G32) {
+                int g = chunk_dot_signed<BITS>(raw[m], asum[asum_index<BITS, MT>(m, chunk_c)]);
+                g = ok ? g : 0;
+                if (G32) {
                     // T2: two neighbouring lanes hold the halves of one group.
                     if (BITS == 2) g += dpp_i32<kDppXor1>(g);
                     const bool writer = (BITS == 2) ? ((c & 1) == 0) : true;
-                    if (writer && chunk < C && row < N && (m0 + m) < M) {
+                    if (writer && ok && (m0 + m) < M) {
                         int32_t *G = reinterpret_cast<int32_t *>(a.out);
                         G[((size_t)(m0 + m) * N + row) * ng + (chunk >> F::kGroupShift)] = g;
                     }
                 } else {
-                    accf[m] += (float)g * cur.sc[u];
+                    accf[m] += (float)g * wsf;
                 }
             }
         }
-
-        if (b == nb - 1 && OUT != OUT_G32) {
+        if (b == nb - 1 && !G32) {
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 const float sum = row_lanes_sum(accf[m], lpr_log2);
                 accf[m] = 0.0f;
-                if (c == 0 && row < N && (m0 + m) < M) {
-                    const float y = sum / a.s[m0 + m];
-                    if (OUT == OUT_F32)
+                if (c == 0 && row_ok && (m0 + m) < M) {
+                    const float y = sum / sdiv[m];
+                    if (a.out_f32)
                         reinterpret_cast<float *>(a.out)[(size_t)(m0 + m) * N + row] = y;
                     else
                         reinterpret_cast<uint16_t *>(a.out)[(size_t)(m0 + m) * N + row] =
@@ -212,9 +242,41 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_dot4_kernel(const GemvArgs a
                 }
             }
         }
-        if (more) cur = nxt;
-        pass = npass;
-        b = nbt;
+    };
+
+    // Batches of all passes form one sequence; two register buffers alternate so
+    // that the loads of batch i+1 are in flight while batch i is consumed.  The
+    // steady-state loop has no conditional loads, which lets the compiler wait
+    // for exactly the loads it needs.
+    const int total = a.passes * nb;
+    auto advance = [&](int &pass, int &b) {
+        if (++b == nb) {
+            b = 0;
+            ++pass;
+        }
+    };
+    int pa = 0, ba = 0;  // position of the batch in `cur`
+    int i = 0;
+    while (i + 2 < total) {
+        int pb = pa, bb = ba;
+        advance(pb, bb);
+        load_batch(nxt, row0 + pb * row_step, bb * U);
+        compute_batch(cur, pa, ba);
+        pa = pb;
+        ba = bb;
+        advance(pa, ba);
+        load_batch(cur, row0 + pa * row_step, ba * U);
+        compute_batch(nxt, pb, bb);
+        i += 2;
+    }
+    if (i + 1 < total) {
+        int pb = pa, bb = ba;
+        advance(pb, bb);
+        load_batch(nxt, row0 + pb * row_step, bb * U);
+        compute_batch(cur, pa, ba);
+        compute_batch(nxt, pb, bb);
+    } else {
+        compute_batch(cur, pa, ba);
     }
 }
 
@@ -228,28 +290,37 @@ struct Tuning {
 };
 
 using KernelFn = void (*)(const GemvArgs);
+constexpr int kBatchKinds = 3;  // U = 1, 2, 4
+constexpr int kVariants = 3;    // 0: bf16 scales, 1: fp16 scales, 2: int32 group sums
 
 template <int BITS>
 struct KernelTable {
-    // [MT-1][out_kind][scale_kind]
-    KernelFn fn[kMaxTile][3][2];
+    KernelFn fn[kMaxTile][kBatchKinds][kVariants];
 };
+
+template <int BITS, int MT, int U, int UI>
+void fill_table_cell(KernelTable<BITS> &t) {
+    t.fn[MT - 1][UI][0] = gemv_dot4_kernel<BITS, MT, U, false, false>;
+    t.fn[MT - 1][UI][1] = gemv_dot4_kernel<BITS, MT, U, false, true>;
+    t.fn[MT - 1][UI][2] = gemv_dot4_kernel<BITS, MT, U, true, false>;
+}
+
+// Register use grows with MT*U (the compiler keeps a whole batch unpacked), so
+// wide token tiles get shorter batches: U <= 4 for MT <= 2, U <= 2 for MT <= 4,
+// U = 1 above.  Cells that are not instantiated stay null.
+constexpr int max_batch_index(int mt) { return mt <= 2 ? 2 : (mt <= 4 ? 1 : 0); }
 
 template <int BITS, int MT>
 void fill_table_row(KernelTable<BITS> &t) {
-    t.fn[MT - 1][OUT_BF16][0] = gemv_dot4_kernel<BITS, MT, OUT_BF16, false>;
-    t.fn[MT - 1][OUT_BF16][1] = gemv_dot4_kernel<BITS, MT, OUT_BF16, true>;
-    t.fn[MT - 1][OUT_F32][0] = gemv_dot4_kernel<BITS, MT, OUT_F32, false>;
-    t.fn[MT - 1][OUT_F32][1] = gemv_dot4_kernel<BITS, MT, OUT_F32, true>;
-    // group sums do not read the scales: one instantiation serves both kinds
-    t.fn[MT - 1][OUT_G32][0] = gemv_dot4_kernel<BITS, MT, OUT_G32, false>;
-    t.fn[MT - 1][OUT_G32][1] = gemv_dot4_kernel<BITS, MT, OUT_G32, false>;
+    fill_table_cell<BITS, MT, 1, 0>(t);
+    if constexpr (max_batch_index(MT) >= 1) fill_table_cell<BITS, MT, 2, 1>(t);
+    if constexpr (max_batch_index(MT) >= 2) fill_table_cell<BITS, MT, 4, 2>(t);
 }
 
 template <int BITS>
 const KernelTable<BITS> &kernel_table() {
     static const KernelTable<BITS> table = [] {
-        KernelTable<BITS> t;
+        KernelTable<BITS> t{};
         fill_table_row<BITS, 1>(t);
         fill_table_row<BITS, 2>(t);
         fill_table_row<BITS, 3>(t);
@@ -291,9 +362,10 @@ int init_device() {
         return 2;
     const KernelTable<BITS> &t = kernel_table<BITS>();
     for (int mt = 0; mt < kMaxTile; ++mt)
-        for (int o = 0; o < 3; ++o)
-            for (int k = 0; k < 2; ++k)
-                if (hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[mt][o][k]),
+        for (int u = 0; u < kBatchKinds; ++u)
+            for (int k = 0; k < kVariants; ++k)
+                if (t.fn[mt][u][k] != nullptr &&
+                    hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[mt][u][k]),
                                         hipFuncAttributeMaxDynamicSharedMemorySize,
                                         max_lds) != hipSuccess)
                     return 2;
@@ -302,7 +374,7 @@ int init_device() {
 }
 
 struct Geometry {
-    int lpr_log2, waves, passes, mt, ntiles, grid_x;
+    int lpr_log2, waves, passes, mt, ntiles, grid_x, batch_index;
     size_t lds;
 };
 
@@ -310,6 +382,15 @@ inline int ilog2(int v) {
     int l = 0;
     while ((1 << (l + 1)) <= v) ++l;
     return l;
+}
+
+template <int BITS>
+size_t lds_bytes(int mt, int C) {
+    static const int words[kMaxTile] = {
+        block_words<BITS, 1>(), block_words<BITS, 2>(), block_words<BITS, 3>(),
+        block_words<BITS, 4>(), block_words<BITS, 5>(), block_words<BITS, 6>(),
+        block_words<BITS, 7>(), block_words<BITS, 8>()};
+    return (size_t)C * words[mt - 1] * 16;
 }
 
 // Picks lanes-per-row, workgroup size and passes for a shape.  The aim is to
@@ -321,16 +402,16 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
     using F = Fmt<BITS>;
     Geometry g{};
     const int C = K / F::kChunkWeights;
-    const size_t per_token = (size_t)K + (size_t)C * 4;
-    int mt_cap = (int)((size_t)lds_limit / per_token);
-    if (mt_cap > kMaxTile) mt_cap = kMaxTile;
+    // largest token tile whose staged blocks fit in LDS
+    int mt_cap = kMaxTile;
+    while (mt_cap >= 1 && lds_bytes<BITS>(mt_cap, C) > (size_t)lds_limit) --mt_cap;
     if (mt_cap < 1) {
         g.mt = 0;
         return g;
     }
     g.ntiles = (M + mt_cap - 1) / mt_cap;
     g.mt = (M + g.ntiles - 1) / g.ntiles;
-    g.lds = (size_t)g.mt * per_token;
+    g.lds = lds_bytes<BITS>(g.mt, C);
 
     int lpr = tu.lanes_per_row;
     if (lpr == 0) {
@@ -347,6 +428,10 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
         lpr = best;
     }
     g.lpr_log2 = ilog2(lpr);
+    // loads per batch: the largest of 4, 2, 1 that wastes no load slot, 4 for long rows
+    const int it = (C + lpr - 1) / lpr;
+    g.batch_index = (it % 4 == 0 || it >= 8) ? 2 : (it % 2 == 0 ? 1 : 0);
+    if (g.batch_index > max_batch_index(g.mt)) g.batch_index = max_batch_index(g.mt);
     const int rpw = 64 >> g.lpr_log2;
     const long wave_passes = ((long)N + rpw - 1) / rpw;
 
@@ -393,8 +478,11 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     args.K = K;
     args.lpr_log2 = g.lpr_log2;
     args.passes = g.passes;
+    args.out_f32 = out_kind == OUT_F32 ? 1 : 0;
+    args.div_magic = (uint32_t)(0x100000000ull / (uint64_t)(4 * (K / Fmt<BITS>::kChunkWeights))) + 1u;
 
-    const KernelFn fn = kernel_table<BITS>().fn[g.mt - 1][out_kind][scale_kind];
+    const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
+    const KernelFn fn = kernel_table<BITS>().fn[g.mt - 1][g.batch_index][variant];
     hipLaunchKernelGGL(fn, dim3(g.grid_x, g.ntiles, 1), dim3(g.waves * 64, 1, 1), g.lds, stream,
                        args);
     return hipGetLastError() == hipSuccess ? 0 : 2;

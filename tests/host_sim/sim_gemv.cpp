@@ -17,15 +17,15 @@ static void run_tile(const int8_t *A, const uint8_t *B, int32_t *G, int m0, int 
     using F = Fmt<BITS>;
     const int C = K / F::kChunkWeights;
     const int ng = K / 128;
-    std::vector<u32x4> act((size_t)MT * F::kUnits * C);
-    std::vector<int> asum((size_t)MT * C);
+    std::vector<u32x4> act((size_t)C * block_words<BITS, MT>());
+    int *asum = reinterpret_cast<int *>(act.data());
     for (int task = 0; task < MT * C; ++task) {
         const int m = task / C, chunk = task - m * C;
         const int msrc = (m0 + m) < M ? (m0 + m) : M - 1;
         std::vector<u32x4> src(F::kUnits);
         std::memcpy(src.data(), A + (size_t)msrc * K + (size_t)chunk * F::kChunkWeights,
                     F::kChunkWeights);
-        asum[(size_t)m * C + chunk] = stage_chunk<BITS>(src.data(), act.data(), m, chunk, C);
+        asum[asum_index<BITS, MT>(m, chunk)] = stage_chunk<BITS, MT>(src.data(), act.data(), m, chunk);
     }
     for (int n = 0; n < N; ++n)
         for (int chunk = 0; chunk < C; ++chunk) {
@@ -33,10 +33,10 @@ static void run_tile(const int8_t *A, const uint8_t *B, int32_t *G, int m0, int 
             std::memcpy(&w, B + (size_t)n * C * 16 + (size_t)chunk * 16, 16);
             int raw[MT];
             for (int m = 0; m < MT; ++m) raw[m] = 0;
-            chunk_dot_raw<BITS, MT>(w, act.data(), chunk, C, raw);
+            chunk_dot_raw<BITS, MT>(w, act.data(), chunk, raw);
             for (int m = 0; m < MT; ++m) {
                 if (m0 + m >= M) continue;
-                const int g = chunk_dot_signed<BITS>(raw[m], asum[(size_t)m * C + chunk]);
+                const int g = chunk_dot_signed<BITS>(raw[m], asum[asum_index<BITS, MT>(m, chunk)]);
                 int32_t *dst = &G[((size_t)(m0 + m) * N + n) * ng + (chunk >> F::kGroupShift)];
                 if (BITS == 2 && (chunk & 1)) *dst += g; else *dst = g;
             }
