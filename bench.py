@@ -26,6 +26,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by a 256 MiB copy), from the
+# two rocprofv3 --pmc runs summarised under profiles/; keyed by width.  Not measured live.
+MEASURED_TRAFFIC_BYTES = {1: (1958.3 + 11.4) * 1024, 4: (2075.5 + 45.7) * 1024,
+                          8: (2185.9 + 91.4) * 1024}
 WIDTHS = (1, 4, 8)
 # name, N, K  (Qwen3-1.7B: hidden 2048, 16 q / 8 kv heads x 128, ffn 6144)
 PROJECTIONS = (
@@ -213,7 +217,8 @@ def main() -> int:
     achieved = bytes_per_launch / (per_width[dom]["us_per_launch"] * 1e-6) / 1e9
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": round(MEASURED_TRAFFIC_BYTES[dom]),
         "kernel": f"gemv_dot4_kernel<BITS=2, MT={dom}, OUT=bf16> (width {dom})",
         "bytes_per_launch": round(bytes_per_launch),
         "us_per_launch": per_width[dom]["us_per_launch"],

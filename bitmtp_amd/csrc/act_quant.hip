@@ -1,6 +1,8 @@
 // libbonsai_actq.so: per-token absmax INT8 activation quantisation for gfx950,
 // the native form of `quant_input` (src/bonsai_sft/gpu/model.py:632-636):
-//   s = 127 / max(max_k |x_k|, 1e-5)           fp32, IEEE division
+//   s = fl(fl(1 / max(max_k |x_k|, 1e-5)) * 127)     two fp32 roundings: PyTorch
+//                                                    evaluates `127.0 / tensor` as
+//                                                    `tensor.reciprocal() * 127.0`
 //   q_k = clamp(round_half_even(fp32(x_k) * s), -128, 127)
 // One workgroup per token; the row is read twice (the second read hits L2) with
 // 16-byte loads and written with 8-byte stores.  HBM-bound: K * (sizeof(x) + 1)
@@ -88,7 +90,8 @@ __global__ void __launch_bounds__(kThreads) act_quant_kernel(const void *x, int8
 #pragma unroll
     for (int w = 1; w < kThreads / 64; ++w) amax = fmaxf(amax, wave_max[w]);
 
-    const float sval = 127.0f / fmaxf(amax, 1e-5f);
+    const float recip = 1.0f / fmaxf(amax, 1e-5f);  // IEEE division, rounded on its own
+    const float sval = recip * 127.0f;
     if (tid == 0) s[m] = sval;
 
     uint2 *qrow = reinterpret_cast<uint2 *>(q + (size_t)m * K);

@@ -278,8 +278,9 @@ def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[tor
 
 def quant_input(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-token absmax INT8 quantisation on the GPU: returns ``(q int8 [..., K],
-    s fp32 [..., 1])`` with ``s = 127 / clamp_min(absmax, 1e-5)`` (reference:
-    model.py:632-636)."""
+    s fp32 [..., 1])`` with ``s = reciprocal(clamp_min(absmax, 1e-5)) * 127`` -- what
+    PyTorch computes for the reference's ``127.0 / absmax.clamp_(min=1e-5)``
+    (model.py:632-636)."""
     if x.dtype not in _X_KIND:
         raise RuntimeError("quant_input: activation must be bfloat16, float16 or float32")
     if not (x.is_cuda and x.is_contiguous()) or x.dim() < 1:

@@ -17,7 +17,7 @@
  *   B   uint8 [N, K/4]      T2: weight k of row n = ((B[n][k/4] >> 2(k%4)) & 3) - 2
  *       uint8 [N, K/8]      Q1: weight k of row n = 2*((B[n][k/8] >> (k%8)) & 1) - 1
  *   ws  16-bit [N, K/128]   one scale per row and 128-wide K group (bf16; the
- *                           *_f16s entry points read IEEE fp16 instead)
+ *                           *_gemv_ex entry points also read IEEE fp16)
  *   s   fp32  [M]           activation MULTIPLIER 127/absmax (the result is divided by it)
  *   C   bf16  [M, N]        C[m][n] = bf16( (sum_g fp32(G[m][n][g]) * ws[n][g]) / s[m] )
  *   G   int32 [M, N, K/128] exact group sums G[m][n][g] = sum_{k in g} A[m][k] * w[n][k]
@@ -102,7 +102,8 @@ void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
 /* ---- activation quantisation (libbonsai_actq.so) ------------------------- */
 /* Per-token symmetric INT8 quantisation, the native form of `quant_input`
  * (src/bonsai_sft/gpu/model.py:632-636, identical copy at :571-575):
- *   s[m] = 127 / max(max_k |x[m][k]|, 1e-5)          (fp32)
+ *   s[m] = fl( fl(1 / max(max_k |x[m][k]|, 1e-5)) * 127 )   (fp32; the reference's
+ *          `127.0 / tensor` is evaluated by PyTorch as `tensor.reciprocal() * 127.0`)
  *   q[m][k] = clamp(round_half_even(fp32(x[m][k]) * s[m]), -128, 127)
  * x_kind selects the element type of x. */
 #define BONSAI_X_BF16 0

@@ -169,7 +169,10 @@ void oracle_pack_q1_g128(const uint16_t *Wlat, uint8_t *B, uint16_t *scales, int
 /* ---- activation quant (model.py:632-636) ------------------------------- */
 
 /* x is the activation already widened to fp32 (x.float() is exact for fp16 and
- * bf16).  s = 127 / max(absmax, 1e-5) in fp32; q = clamp(rint(x*s), -128, 127). */
+ * bf16).  The reference writes `127.0 / absmax.clamp_(min=1e-5)`; PyTorch evaluates
+ * a Python scalar divided by a tensor as `tensor.reciprocal() * scalar`
+ * (Tensor.__rtruediv__), i.e. TWO fp32 roundings, so
+ *     s = fl( fl(1 / max(absmax, 1e-5)) * 127 ),   q = clamp(rint(fl(x*s)), -128, 127). */
 void oracle_act_quant(const float *X, int8_t *Q, float *S, int M, int K) {
     for (int m = 0; m < M; ++m) {
         const float *x = X + (size_t)m * K;
@@ -179,7 +182,8 @@ void oracle_act_quant(const float *X, int8_t *Q, float *S, int M, int K) {
             if (a > amax) amax = a;
         }
         if (amax < 1e-5f) amax = 1e-5f;
-        float s = 127.0f / amax;
+        volatile float recip = 1.0f / amax; /* kept as its own rounding step */
+        float s = recip * 127.0f;
         S[m] = s;
         for (int k = 0; k < K; ++k) {
             float r = rintf(x[k] * s); /* default rounding mode: half to even */

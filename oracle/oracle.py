@@ -171,7 +171,8 @@ def np_unpack(B: np.ndarray, bits: int) -> np.ndarray:
 def np_act_quant(X: np.ndarray):
     Xf = np.asarray(X, dtype=np.float32)
     amax = np.maximum(np.abs(Xf).max(axis=-1, keepdims=True), np.float32(1e-5))
-    s = (np.float32(127.0) / amax).astype(np.float32)
+    recip = (np.float32(1.0) / amax).astype(np.float32)  # torch: scalar / tensor = reciprocal * scalar
+    s = (recip * np.float32(127.0)).astype(np.float32)
     q = np.clip(np.rint((Xf * s).astype(np.float32)), -128, 127).astype(np.int8)
     return q, s.reshape(-1)
 

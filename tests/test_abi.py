@@ -1,0 +1,59 @@
+"""The C-ABI libraries load without a GPU and export every entry point that
+include/bonsai_gemv.h declares (no compute call is made here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "bonsai_gemv.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(?:int|void)\s+([a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def libs():
+    from bitmtp_amd import build, ops
+    build.build_all(verbose=False)  # compiles only what is missing or out of date
+    paths = [ops.t2_lib_path(), ops.q1_lib_path(), ops.actq_lib_path()]
+    assert all(os.path.exists(p) for p in paths)
+    return [ctypes.CDLL(p) for p in paths]
+
+
+def test_header_declares_the_drop_in_symbols():
+    names = declared_functions()
+    for required in ("t2g128_int8xint2_linear", "q1g128_int8xint1_linear", "q1g128_w1a16_linear"):
+        assert required in names
+
+
+def test_every_declared_symbol_is_exported(libs):
+    for name in declared_functions():
+        owners = [lib for lib in libs if hasattr(lib, name)]
+        assert len(owners) == 1, f"{name} exported by {len(owners)} libraries"
+
+
+def test_reference_loader_view_of_the_libraries(libs):
+    """What the reference's ctypes loaders touch (src/bonsai_sft/gpu/model.py:70-93,
+    206-219): both Q1 symbols in libbonsai_q1.so, the T2 symbol in libbonsai_t2.so."""
+    t2, q1, _ = libs
+    assert hasattr(t2, "t2g128_int8xint2_linear")
+    assert hasattr(q1, "q1g128_int8xint1_linear") and hasattr(q1, "q1g128_w1a16_linear")
+    from bitmtp_amd import ops
+    assert ops.t2_lib_path().endswith(os.path.join("t2g128_kernels", "libbonsai_t2.so"))
+    assert ops.q1_lib_path().endswith(os.path.join("q1g128_kernels", "libbonsai_q1.so"))
+
+
+def test_python_binding_sets_argtypes():
+    from bitmtp_amd import ops
+    ops.load_t2_kernel()
+    ops.load_q1_kernel()
+    ops.load_actq_kernel()
+    assert len(ops.t2_lib().t2g128_int8xint2_linear.argtypes) == 9
+    assert ops.t2_lib().t2g128_int8xint2_linear.restype is None
+    assert len(ops.q1_lib().q1g128_w1a16_linear.argtypes) == 8
+    assert len(ops.t2_lib().t2g128_gemv_ex.argtypes) == 11
