@@ -36,15 +36,6 @@
 #define BONSAI_HD inline
 #endif
 
-// Scheduling fence for the device compiler: nothing is moved across it.  Used to
-// bound how many LDS reads are hoisted ahead of the arithmetic that consumes
-// them (each costs four registers).
-#if defined(__HIP_DEVICE_COMPILE__)
-#define BONSAI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-#else
-#define BONSAI_SCHED_FENCE() ((void)0)
-#endif
-
 namespace bonsai {
 
 struct alignas(16) u32x4 {
@@ -204,6 +195,72 @@ template <int BITS>
 BONSAI_HD int chunk_dot_signed(int raw, int asum) {
     return BITS == 2 ? raw - 2 * asum : 2 * raw - asum;
 }
+
+// ---------------------------------------------------------------------------
+// Matrix-core (MFMA) path: operand slots
+// ---------------------------------------------------------------------------
+// v_mfma_i32_16x16x64_i8 contracts 64 K-slots per instruction.  Lane l supplies,
+// for matrix row/column l % 16, the 16 slots of K-block kb = l / 16 as four
+// registers of four bytes, and slot (kb, reg, byte) of one operand meets the
+// same slot of the other.  A 128-weight scale group is two MFMAs (t = 0, 1)
+// into one accumulator.  Lane kb owns weights 32*kb .. 32*kb+31 of the group:
+//   T2: packed dwords 2kb and 2kb+1 of the group's eight; MFMA t takes dword
+//       2kb+t unpacked as u_j = (p >> 2j) & 0x03030303:
+//           slot (reg j, byte b) = weight 32kb + 16t + 4b + j
+//   Q1: packed dword kb of the group's four; u_j = (p >> j) & 0x01010101 and
+//       MFMA t takes u_{4t} .. u_{4t+3}:
+//           slot (reg j, byte b) = weight 32kb + 8b + 4t + j
+// In both formats the activation operand for (kb, t) is staged unit 2kb+t of
+// the group, holding the activations of those weights in (reg, byte) order --
+// the same 4x4 byte transposes the dot4 path stages.
+template <int BITS>
+BONSAI_HD void mfma_unpack(uint32_t p0, uint32_t p1, uint32_t b0[4], uint32_t b1[4]) {
+    if (BITS == 2) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            b0[j] = (p0 >> (2 * j)) & 0x03030303u;
+            b1[j] = (p1 >> (2 * j)) & 0x03030303u;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            b0[j] = (p0 >> j) & 0x01010101u;
+            b1[j] = (p0 >> (4 + j)) & 0x01010101u;
+        }
+    }
+}
+
+// Staged activations of the MFMA path: token-major, one 16-byte unit per (group,
+// kb, t) in natural K order, each token padded by one unit so that the sixteen
+// tokens a ds_read_b128 touches fall into distinct bank groups.
+BONSAI_HD int mfma_token_words(int K) { return K / 16 + 1; }
+
+// Natural-order activations per staging quarter: 16 (T2) or 32 (Q1).
+template <int BITS>
+BONSAI_HD constexpr int mfma_quarter_bytes() { return BITS == 2 ? 16 : 32; }
+
+// Stage quarter q of one token (src = the quarter's natural-order activations);
+// returns the sum of its activations.
+template <int BITS>
+BONSAI_HD int mfma_stage_quarter(const u32x4 *src, u32x4 *act_token, int q) {
+    if (BITS == 2) {
+        const u32x4 in = src[0];
+        act_token[q] = transpose4x4_bytes(in.x, in.y, in.z, in.w);
+        return sum4_i8(in.x) + sum4_i8(in.y) + sum4_i8(in.z) + sum4_i8(in.w);
+    } else {
+        const u32x4 lo = src[0], hi = src[1];
+        act_token[2 * q] = transpose4x4_bytes(lo.x, lo.z, hi.x, hi.z);
+        act_token[2 * q + 1] = transpose4x4_bytes(lo.y, lo.w, hi.y, hi.w);
+        return sum4_i8(lo.x) + sum4_i8(lo.y) + sum4_i8(lo.z) + sum4_i8(lo.w) +
+               sum4_i8(hi.x) + sum4_i8(hi.y) + sum4_i8(hi.z) + sum4_i8(hi.w);
+    }
+}
+
+// Offset-removal term stored per (group, token): G = mfma_scale * D + corr.
+template <int BITS>
+BONSAI_HD int mfma_corr(int group_asum) { return BITS == 2 ? -2 * group_asum : -group_asum; }
+template <int BITS>
+BONSAI_HD int mfma_group_sum(int d, int corr) { return (BITS == 2 ? d : 2 * d) + corr; }
 
 }  // namespace bonsai
 #endif  // BONSAI_GEMV_CORE_H

@@ -340,6 +340,7 @@ template <int BITS>
 struct LibState {
     Tuning tuning;
     int lds_limit[kMaxDevices] = {};  // 0 = device not initialised yet
+    bool mfma_ready[kMaxDevices] = {};
 };
 
 template <int BITS>
@@ -448,23 +449,12 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
     return g;
 }
 
+// Launches the dot4 kernel for a validated shape on an initialised device.
 template <int BITS>
-int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
-                int M, int N, int K, int out_kind, int scale_kind, hipStream_t stream) {
-    if (A == nullptr || B == nullptr || out == nullptr) return 1;
-    if (out_kind < 0 || out_kind > 2 || scale_kind < 0 || scale_kind > 1) return 1;
-    if (out_kind != OUT_G32 && (s == nullptr || ws == nullptr)) return 1;
-    if (M < 1 || N < 1 || K < kGroup || K % kGroup != 0) return 1;
-    if ((long)M * N > 0x7fffffffL / 2) return 1;  // row indices are 32-bit
-
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 2;
-    LibState<BITS> &st = lib_state<BITS>();
-    if (st.lds_limit[dev] == 0) {
-        const int rc = init_device<BITS>();
-        if (rc != 0) return rc;
-    }
-    const Geometry g = pick_geometry<BITS>(M, N, K, st.lds_limit[dev], st.tuning);
+int launch_gemv_dot4(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
+                     int M, int N, int K, int out_kind, int scale_kind, int lds_limit,
+                     hipStream_t stream) {
+    const Geometry g = pick_geometry<BITS>(M, N, K, lds_limit, lib_state<BITS>().tuning);
     if (g.mt == 0) return 1;  // one token of K activations does not fit in LDS
 
     GemvArgs args;

@@ -1,7 +1,7 @@
 // libbonsai_q1.so: C ABI of the Q1-g128 (sign, 1 bit) W1A8 GEMV for gfx950.
 // Entry points are declared in include/bonsai_gemv.h; the drop-in one replaces
 // src/bonsai_sft/gpu/q1g128_kernels/q1g128_kernels_block8.cu:118-241.
-#include "packed_gemv.hip.h"
+#include "gemv_dispatch.hip.h"
 
 #include "../../include/bonsai_gemv.h"
 
@@ -78,13 +78,20 @@ void q1g128_w1a16_linear(const void *A, const int8_t *B, void *C, const void *ws
                        K);
 }
 
-int q1g128_init(void) { return init_device<1>(); }
+int q1g128_init(void) { return init_all_kernels<1>(); }
 
 void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes) {
     Tuning &t = lib_state<1>().tuning;
     t.lanes_per_row = lanes_per_row;
     t.waves_per_wg = waves_per_wg;
     t.passes = passes;
+}
+
+void q1g128_set_mfma_tuning(int min_width, int row_tiles, int k_split) {
+    MfmaTuning &t = mfma_tuning<1>();
+    t.min_width = min_width;
+    t.row_tiles = row_tiles;
+    t.k_split = k_split;
 }
 
 int q1g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,

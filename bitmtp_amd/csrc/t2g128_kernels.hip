@@ -1,7 +1,7 @@
 // libbonsai_t2.so: C ABI of the T2-g128 (ternary, 2-bit codes) W2A8 GEMV for
 // gfx950.  Entry points are declared in include/bonsai_gemv.h; the drop-in one
 // replaces src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:123-148.
-#include "packed_gemv.hip.h"
+#include "gemv_dispatch.hip.h"
 
 #include "../../include/bonsai_gemv.h"
 
@@ -9,13 +9,20 @@ using namespace bonsai;
 
 extern "C" {
 
-int t2g128_init(void) { return init_device<2>(); }
+int t2g128_init(void) { return init_all_kernels<2>(); }
 
 void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes) {
     Tuning &t = lib_state<2>().tuning;
     t.lanes_per_row = lanes_per_row;
     t.waves_per_wg = waves_per_wg;
     t.passes = passes;
+}
+
+void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split) {
+    MfmaTuning &t = mfma_tuning<2>();
+    t.min_width = min_width;
+    t.row_tiles = row_tiles;
+    t.k_split = k_split;
 }
 
 int t2g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,

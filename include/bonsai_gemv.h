@@ -99,6 +99,12 @@ int q1g128_init(void);
 void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
 void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
 
+/* The same for the matrix-core kernel that serves widths >= min_width: smallest
+ * width it takes (a value above any M disables it), 16-row tiles per wave (1, 2
+ * or 4) and waves of a workgroup splitting K (1, 2 or 4).  Zero = built-in choice. */
+void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split);
+void q1g128_set_mfma_tuning(int min_width, int row_tiles, int k_split);
+
 /* ---- activation quantisation (libbonsai_actq.so) ------------------------- */
 /* Per-token symmetric INT8 quantisation, the native form of `quant_input`
  * (src/bonsai_sft/gpu/model.py:632-636, identical copy at :571-575):

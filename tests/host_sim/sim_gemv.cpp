@@ -59,3 +59,64 @@ extern "C" int sim_group_sums(const int8_t *A, const uint8_t *B, int32_t *G, int
     }
     return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Matrix-core path.  The MFMA is modelled by its contract: slot (kb, reg, byte) of
+// the token operand meets the same slot of the weight operand, D[token][row] is
+// the sum over the 64 slots.  Everything else -- activation staging order, the
+// correction terms, which packed dword a lane unpacks for which of the two MFMAs
+// of a group -- is the kernel's own code from gemv_core.h.
+// ---------------------------------------------------------------------------
+template <int BITS>
+static void run_mfma(const int8_t *A, const uint8_t *B, int32_t *G, int M, int N, int K) {
+    const int ng = K / 128;
+    const int tw = mfma_token_words(K);
+    constexpr int QB = mfma_quarter_bytes<BITS>();
+    constexpr int QPG = 128 / QB;
+    std::vector<u32x4> act((size_t)M * tw);
+    std::vector<int> corr((size_t)ng * M);
+    for (int tok = 0; tok < M; ++tok)
+        for (int g = 0; g < ng; ++g) {
+            int sum = 0;
+            for (int qi = 0; qi < QPG; ++qi) {
+                const int q = g * QPG + qi;
+                u32x4 src[2];
+                std::memcpy(src, A + (size_t)tok * K + (size_t)q * QB, QB);
+                sum += mfma_stage_quarter<BITS>(src, act.data() + (size_t)tok * tw, q);
+            }
+            corr[(size_t)g * M + tok] = mfma_corr<BITS>(sum);
+        }
+    const int row_bytes = K * BITS / 8;
+    for (int n = 0; n < N; ++n)
+        for (int g = 0; g < ng; ++g)
+            for (int tok = 0; tok < M; ++tok) {
+                int d = 0;
+                for (int kb = 0; kb < 4; ++kb) {
+                    uint32_t p0, p1 = 0;
+                    const uint8_t *grp = B + (size_t)n * row_bytes + (size_t)g * (128 * BITS / 8);
+                    if (BITS == 2) {
+                        std::memcpy(&p0, grp + kb * 8, 4);
+                        std::memcpy(&p1, grp + kb * 8 + 4, 4);
+                    } else {
+                        std::memcpy(&p0, grp + kb * 4, 4);
+                    }
+                    uint32_t b0[4], b1[4];
+                    mfma_unpack<BITS>(p0, p1, b0, b1);
+                    const u32x4 a0 = act[(size_t)tok * tw + g * 8 + 2 * kb];
+                    const u32x4 a1 = act[(size_t)tok * tw + g * 8 + 2 * kb + 1];
+                    const uint32_t av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
+                    for (int j = 0; j < 4; ++j) {
+                        d = dot4_i8(av0[j], b0[j], d);
+                        d = dot4_i8(av1[j], b1[j], d);
+                    }
+                }
+                G[((size_t)tok * N + n) * ng + g] = mfma_group_sum<BITS>(d, corr[(size_t)g * M + tok]);
+            }
+}
+
+extern "C" int sim_group_sums_mfma(const int8_t *A, const uint8_t *B, int32_t *G, int M, int N, int K,
+                                   int bits) {
+    if (K % 128 != 0) return 1;
+    if (bits == 2) run_mfma<2>(A, B, G, M, N, K); else run_mfma<1>(A, B, G, M, N, K);
+    return 0;
+}

@@ -23,6 +23,8 @@ def sim():
     L = ctypes.CDLL(OUT)
     L.sim_group_sums.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 5
     L.sim_group_sums.restype = ctypes.c_int
+    L.sim_group_sums_mfma.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4
+    L.sim_group_sums_mfma.restype = ctypes.c_int
     return L
 
 
@@ -36,4 +38,17 @@ def test_lane_arithmetic_matches_oracle(oracle, sim, bits, M, N, K, mt):
     G = np.zeros((M, N, K // 128), dtype=np.int32)
     rc = sim.sim_group_sums(A.ctypes.data, B.ctypes.data, G.ctypes.data, M, N, K, bits, mt)
     assert rc == 0
+    assert np.array_equal(G, oracle.c_group_sums(A, B, bits))
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+@pytest.mark.parametrize("M,N,K", [(1, 4, 128), (3, 5, 512), (16, 3, 2560), (9, 2, 1024)])
+def test_mfma_slot_mapping_matches_oracle(oracle, sim, bits, M, N, K):
+    """Matrix-core path: staged operand order, per-MFMA dword choice and correction
+    terms reproduce the exact group sums (the MFMA itself is modelled slot by slot)."""
+    rng = np.random.default_rng(M * 7 + N * 3 + K + bits)
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(0, 256, size=(N, K * bits // 8), dtype=np.uint8)
+    G = np.zeros((M, N, K // 128), dtype=np.int32)
+    assert sim.sim_group_sums_mfma(A.ctypes.data, B.ctypes.data, G.ctypes.data, M, N, K, bits) == 0
     assert np.array_equal(G, oracle.c_group_sums(A, B, bits))
