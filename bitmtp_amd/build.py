@@ -30,6 +30,9 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed fp32 VALU forms are kept out of generated code on this target
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results go to ordinary VGPRs: the scale-accumulate epilogue consumes them
+    # at once and v_accvgpr_read copies would cost four VALU slots per tile
+    "-mllvm", "--amdgpu-mfma-vgpr-form",
 ]
 
 

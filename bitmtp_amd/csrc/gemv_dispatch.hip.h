@@ -1,12 +1,14 @@
 // Entry-point logic shared by libbonsai_t2.so and libbonsai_q1.so: argument
-// checks, one-time device set-up and the choice between the two kernels --
-// the dot4 kernel (packed_gemv.hip.h) for a single token and for shapes the
-// matrix-core kernel does not take, the MFMA kernel (gemv_mfma.hip.h) from
-// `min_width` tokens on.  Replaces the if-chain over registered (M, N, K) of the
+// checks, one-time device set-up and the choice among the three kernels -- the
+// FP4 x FP8 matrix-core kernel (gemv_fp4.hip.h) whenever its staged activations
+// fit in LDS as one token tile, the int8 matrix-core kernel (gemv_mfma.hip.h)
+// for long rows at wide blocks, and the dot4 kernel (packed_gemv.hip.h) for
+// shapes neither takes (K not a multiple of 512, unaligned operands).  Replaces the if-chain over registered (M, N, K) of the
 // reference (src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:94-148).
 #ifndef BONSAI_GEMV_DISPATCH_HIP_H
 #define BONSAI_GEMV_DISPATCH_HIP_H
 
+#include "gemv_fp4.hip.h"
 #include "gemv_mfma.hip.h"
 #include "packed_gemv.hip.h"
 
@@ -24,9 +26,84 @@ int init_all_kernels() {
     if (!st.mfma_ready[dev]) {
         const int rc2 = mfma_init_device<BITS>(st.lds_limit[dev]);
         if (rc2 != 0) return rc2;
+        const int rc3 = fp4_init_device<BITS>(st.lds_limit[dev]);
+        if (rc3 != 0) return rc3;
         st.mfma_ready[dev] = true;
     }
     return 0;
+}
+
+// Launches one of the two matrix-core kernels.  Returns -1 when the shape does not
+// fit (the caller falls back), 0 on success, 2 on a launch error.  `single_tile`
+// refuses shapes whose tokens would need more than ceil(M/16) token tiles, i.e.
+// a second pass over the weights.
+template <int BITS>
+int launch_matrix_core(bool fp4, bool single_tile, const int8_t *A, const uint8_t *B, void *out,
+                       const float *s, const void *ws, int M, int N, int K, int out_kind,
+                       int scale_kind, int lds_limit, hipStream_t stream) {
+    const MfmaTuning &tu = mfma_tuning<BITS>();
+    auto lds_for = [&](int ri, int mt) {
+        return fp4 ? fp4_lds_for<BITS>(ri, mt, K) : mfma_lds_for<BITS>(ri, mt, K);
+    };
+    int ntok_tiles = (M + kMfmaTokens - 1) / kMfmaTokens;
+    int mt = (M + ntok_tiles - 1) / ntok_tiles;
+    while (lds_for(0, mt) > (size_t)lds_limit) {
+        if (single_tile || mt == 1) return -1;
+        ++ntok_tiles;
+        mt = (M + ntok_tiles - 1) / ntok_tiles;
+    }
+
+    // K split among the waves of a workgroup for short matrices, more row tiles per
+    // wave and several row blocks per workgroup for long ones.
+    int ks = tu.k_split;
+    int R = tu.row_tiles;
+    const int ntiles = K / 512;
+    if (ks == 0)
+        ks = (ntiles % 4 == 0 && (long)N * 4 <= 16384) ? 4
+             : ((ntiles % 2 == 0 && (long)N * 2 <= 16384) ? 2 : 1);
+    if (ks != 1 && ks != 2 && ks != 4) ks = 1;
+    if (ks > ntiles) ks = 1;
+    if (R == 0) {
+        const long wgs1 = ((long)N + 16 * (4 / ks) - 1) / (16 * (4 / ks));  // workgroups at R = 1
+        R = wgs1 >= 8192 ? 4 : (wgs1 >= 2048 ? 2 : 1);
+    }
+    int ri = R >= 4 ? 2 : (R >= 2 ? 1 : 0);
+    while (ri > 0 && lds_for(ri, mt) > (size_t)lds_limit) --ri;
+    R = 1 << ri;
+
+    int passes = 1;
+    if (ks == 1) {
+        passes = tu.passes;
+        if (passes == 0) {
+            const long blocks = ((long)N + 64 * R - 1) / (64 * R);
+            passes = blocks >= 4096 ? 4 : (blocks >= 2048 ? 2 : 1);
+        }
+        if (passes < 1) passes = 1;
+    }
+
+    MfmaArgs args;
+    args.A = A;
+    args.B = B;
+    args.out = out;
+    args.s = s;
+    args.ws = reinterpret_cast<const uint16_t *>(ws);
+    args.M = M;
+    args.N = N;
+    args.K = K;
+    args.mt = mt;
+    args.ks_log2 = ks == 4 ? 2 : (ks == 2 ? 1 : 0);
+    args.out_f32 = out_kind == OUT_F32 ? 1 : 0;
+    args.passes = passes;
+    const int per_token = fp4 ? K / 32 : K / mfma_quarter_bytes<BITS>();  // staging tasks per token
+    args.div_magic = (uint32_t)(0x100000000ull / (uint64_t)per_token) + 1u;
+
+    const int rows_per_wg = 16 * R * (4 / ks) * passes;
+    const int grid_x = (N + rows_per_wg - 1) / rows_per_wg;
+    const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
+    const MfmaKernelFn fn = fp4 ? fp4_table<BITS>().fn[ri][variant] : mfma_table<BITS>().fn[ri][variant];
+    hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(kMfmaThreads, 1, 1), lds_for(ri, mt),
+                       stream, args);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
 template <int BITS>
@@ -50,8 +127,13 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     const MfmaTuning &mtu = mfma_tuning<BITS>();
     const int min_width = mtu.min_width > 0 ? mtu.min_width : kDefaultMfmaMinWidth;
     if (M >= min_width && mfma_shape_ok(B, out_kind == OUT_G32 ? nullptr : ws, K)) {
-        const int rc = launch_gemv_mfma<BITS>(A, B, out, s, ws, M, N, K, out_kind, scale_kind,
-                                              lds_limit, stream);
+        int rc = -1;
+        if (mtu.engine != 1)
+            rc = launch_matrix_core<BITS>(true, mtu.engine == 0, A, B, out, s, ws, M, N, K, out_kind,
+                                          scale_kind, lds_limit, stream);
+        if (rc < 0 && mtu.engine != 2)
+            rc = launch_matrix_core<BITS>(false, false, A, B, out, s, ws, M, N, K, out_kind,
+                                          scale_kind, lds_limit, stream);
         if (rc >= 0) return rc;
     }
     return launch_gemv_dot4<BITS>(A, B, out, s, ws, M, N, K, out_kind, scale_kind, lds_limit,

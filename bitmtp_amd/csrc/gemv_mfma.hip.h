@@ -5,9 +5,9 @@
 // rows x one 128-wide group are unpacked once into the B operand of two
 // v_mfma_i32_16x16x64_i8 and multiplied with up to 16 tokens at the cost the
 // dot4 path pays for one: per group and 16 rows, 14 (T2) / 15 (Q1) unpack
-// operations plus 13 for the exact-int32 -> fp32 scale-accumulate.
+// operations plus 9 for the exact-int32 -> fp32 scale-accumulate.
 //
-//   D[token][row] (int32, exact) = sum over the group's 128 slots;  G = D (+ corr)
+//   G[token][row] (int32, exact) = MFMA over the group's 128 slots, offset term as C input
 //   acc[token][row] += fp32(G) * ws[row][group]                      (fp32)
 //
 // Data movement per wave: R tiles of 16 rows.  Weights are read from HBM with
@@ -40,6 +40,8 @@ struct MfmaArgs {
     int mt;        // tokens per token tile (<= 16); grid.y tiles cover M
     int ks_log2;   // log2 of the waves that split K inside a workgroup (0, 1, 2)
     int out_f32;
+    int passes;          // row blocks a workgroup walks through (1 unless ks_log2 == 0)
+    uint32_t div_magic;  // floor(2^32 / quarters-per-token) + 1: staging task -> token
 };
 
 template <int BITS>
@@ -84,7 +86,8 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel(const MfmaArgs 
     const int rws = 4 >> a.ks_log2;        // row-waves per workgroup
     const int m0 = blockIdx.y * a.mt;
     const int mt = (M - m0) < a.mt ? (M - m0) : a.mt;  // valid tokens of this tile
-    const int n0 = ((int)blockIdx.x * rws + rw) * (16 * R);
+    const int pass_rows = rws * 16 * R;  // rows one pass of the workgroup covers
+    const int n_first = (int)blockIdx.x * a.passes * pass_rows + rw * (16 * R);
 
     // ---- LDS carve-up
     const int tw = mfma_token_words(K);
@@ -110,7 +113,7 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel(const MfmaArgs 
         u32x4 w[R][MF::kLoads];
         uint2 sc[R];  // four bf16/fp16 scales of this lane's row
     };
-    auto load_tile = [&](TileRegs &tr, int kt) {
+    auto load_tile = [&](TileRegs &tr, int n0, int kt) {
 #pragma unroll
         for (int rt = 0; rt < R; ++rt) {
 #pragma unroll
@@ -143,7 +146,7 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel(const MfmaArgs 
     };
 
     TileRegs cur;
-    if (t_begin < t_end) load_tile(cur, t_begin);
+    if (t_begin < t_end) load_tile(cur, n_first, t_begin);
 
     float sdiv[4];
     if (!G32) {
@@ -154,21 +157,39 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel(const MfmaArgs 
         }
     }
 
-    // ---- stage the token tile (operand order) and the per-group correction terms
+    // ---- stage the token tile (operand order) and the per-group correction terms.
+    // Four quarter tasks per thread and round: their loads go out together.
     {
         constexpr int QB = mfma_quarter_bytes<BITS>();
+        constexpr int QW = QB / 16;       // 16-byte words per quarter
         constexpr int QPG = kGroup / QB;  // quarters per group: 8 (T2) or 4 (Q1)
+        constexpr int kSt = 4;
         const int qn = K / QB;            // quarters per token
-        for (int task = tid; task < mt * qn; task += kMfmaThreads) {
-            const int tok = task / qn;
-            const int q = task - tok * qn;
-            const u32x4 *src =
-                reinterpret_cast<const u32x4 *>(a.A + (size_t)(m0 + tok) * K + (size_t)q * QB);
-            int sum = mfma_stage_quarter<BITS>(src, act + (size_t)tok * tw, q);
-            sum += dpp_i32<kDppXor1>(sum);
-            sum += dpp_i32<kDppXor2>(sum);
-            if (QPG == 8) sum += dpp_i32<kDppHalfMirror>(sum);
-            if ((q & (QPG - 1)) == 0) corr[(q / QPG) * kMfmaTokens + tok] = mfma_corr<BITS>(sum);
+        const int ntask = mt * qn;
+        for (int base = tid; base < ntask; base += kSt * kMfmaThreads) {
+            u32x4 in[kSt][QW];
+            int tok[kSt], q[kSt];
+#pragma unroll
+            for (int i = 0; i < kSt; ++i) {
+                int task = base + i * kMfmaThreads;
+                task = task < ntask ? task : ntask - 1;  // clamped duplicates are not written
+                tok[i] = (int)__umulhi((uint32_t)task, a.div_magic);  // task / qn
+                q[i] = task - tok[i] * qn;
+                const u32x4 *src = reinterpret_cast<const u32x4 *>(
+                    a.A + (size_t)(m0 + tok[i]) * K + (size_t)q[i] * QB);
+#pragma unroll
+                for (int w = 0; w < QW; ++w) in[i][w] = src[w];
+            }
+#pragma unroll
+            for (int i = 0; i < kSt; ++i) {
+                if (base + i * kMfmaThreads >= ntask) break;  // whole lane groups drop out together
+                int sum = mfma_stage_quarter<BITS>(in[i], act + (size_t)tok[i] * tw, q[i]);
+                sum += dpp_i32<kDppXor1>(sum);
+                sum += dpp_i32<kDppXor2>(sum);
+                if (QPG == 8) sum += dpp_i32<kDppHalfMirror>(sum);
+                if ((q[i] & (QPG - 1)) == 0)
+                    corr[(q[i] / QPG) * kMfmaTokens + tok[i]] = mfma_corr<BITS>(sum);
+            }
         }
     }
     __syncthreads();
@@ -183,94 +204,100 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel(const MfmaArgs 
     const int a_tok = op_row < mt ? op_row : mt - 1;
     const u32x4 *act_lane = act + (size_t)a_tok * tw + 2 * kb;
 
-    for (int kt = t_begin; kt < t_end; ++kt) {
-        park_tile(cur);
-        TileRegs nxt;
-        const bool more = kt + 1 < t_end;
-        if (more) load_tile(nxt, kt + 1);
+    for (int pass = 0; pass < a.passes; ++pass) {
+        const int n0 = n_first + pass * pass_rows;
+        for (int kt = t_begin; kt < t_end; ++kt) {
+            park_tile(cur);
+            TileRegs nxt;
+            // next tile of this row block, or the first tile of the next row block
+            const bool last_kt = kt + 1 == t_end;
+            const bool more = !last_kt || pass + 1 < a.passes;
+            if (more) load_tile(nxt, last_kt ? n0 + pass_rows : n0, last_kt ? t_begin : kt + 1);
 
 #pragma unroll
-        for (int gi = 0; gi < kMfmaGroupsPerTile; ++gi) {
-            const int g = kt * kMfmaGroupsPerTile + gi;
-            const u32x4 a0 = act_lane[g * 8];      // unit 8g + 2kb
-            const u32x4 a1 = act_lane[g * 8 + 1];  // unit 8g + 2kb + 1
-            const v4i va0 = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w};
-            const v4i va1 = {(int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
-            const int4 cr = *reinterpret_cast<const int4 *>(corr + g * kMfmaTokens + 4 * kb);
-            const int crr[4] = {cr.x, cr.y, cr.z, cr.w};
+            for (int gi = 0; gi < kMfmaGroupsPerTile; ++gi) {
+                const int g = kt * kMfmaGroupsPerTile + gi;
+                const u32x4 a0 = act_lane[g * 8];      // unit 8g + 2kb
+                const u32x4 a1 = act_lane[g * 8 + 1];  // unit 8g + 2kb + 1
+                const v4i va0 = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w};
+                const v4i va1 = {(int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                // offset-removal terms of tokens 4kb..4kb+3: the accumulator input
+                const int4 cr = *reinterpret_cast<const int4 *>(corr + g * kMfmaTokens + 4 * kb);
+                const v4i vcr = {cr.x, cr.y, cr.z, cr.w};
 #pragma unroll
-            for (int rt = 0; rt < R; ++rt) {
-                const unsigned char *src = wt + (rt * 16 + op_row) * MF::kPitch;
-                uint32_t p0, p1;
-                if (BITS == 2) {
-                    const uint2 pp = *reinterpret_cast<const uint2 *>(src + gi * 32 + kb * 8);
-                    p0 = pp.x;
-                    p1 = pp.y;
-                } else {
-                    p0 = *reinterpret_cast<const uint32_t *>(src + gi * 16 + kb * 4);
-                    p1 = 0;
-                }
-                uint32_t b0[4], b1[4];
-                mfma_unpack<BITS>(p0, p1, b0, b1);
-                const v4i vb0 = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3]};
-                const v4i vb1 = {(int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
-                v4i d = {0, 0, 0, 0};
-                d = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, vb0, d, 0, 0, 0);
-                d = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, vb1, d, 0, 0, 0);
-                // d[r]: token 4*kb + r, weight row op_row of row tile rt
-                if (G32) {
-                    const int row = n0 + rt * 16 + op_row;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int tok = 4 * kb + r;
-                        if (row < N && tok < mt)
-                            reinterpret_cast<int32_t *>(a.out)[((size_t)(m0 + tok) * N + row) * G + g] =
-                                mfma_group_sum<BITS>(d[r], crr[r]);
+                for (int rt = 0; rt < R; ++rt) {
+                    const unsigned char *src = wt + (rt * 16 + op_row) * MF::kPitch;
+                    uint32_t p0, p1;
+                    if (BITS == 2) {
+                        const uint2 pp = *reinterpret_cast<const uint2 *>(src + gi * 32 + kb * 8);
+                        p0 = pp.x;
+                        p1 = pp.y;
+                    } else {
+                        p0 = *reinterpret_cast<const uint32_t *>(src + gi * 16 + kb * 4);
+                        p1 = 0;
                     }
-                } else {
-                    const uint32_t raw = (gi & 2) ? cur.sc[rt].y : cur.sc[rt].x;
-                    const float wsf = scale_to_f32<SF16>((uint16_t)((gi & 1) ? (raw >> 16) : (raw & 0xffffu)));
+                    uint32_t b0[4], b1[4];
+                    mfma_unpack<BITS>(p0, p1, b0, b1);
+                    const v4i vb0 = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3]};
+                    const v4i vb1 = {(int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+                    v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, vb0, vcr, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, vb1, d, 0, 0, 0);
+                    // d[r]: exact group sum of token 4*kb + r and weight row op_row of tile rt
+                    if (G32) {
+                        const int row = n0 + rt * 16 + op_row;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        acc[rt][r] += (float)mfma_group_sum<BITS>(d[r], crr[r]) * wsf;
+                        for (int r = 0; r < 4; ++r) {
+                            const int tok = 4 * kb + r;
+                            if (row < N && tok < mt)
+                                reinterpret_cast<int32_t *>(
+                                    a.out)[((size_t)(m0 + tok) * N + row) * G + g] = d[r];
+                        }
+                    } else {
+                        const uint32_t raw = (gi & 2) ? cur.sc[rt].y : cur.sc[rt].x;
+                        const float wsf = scale_to_f32<SF16>(
+                            (uint16_t)((gi & 1) ? (raw >> 16) : (raw & 0xffffu)));
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[rt][r] += (float)d[r] * wsf;
+                    }
                 }
             }
+            if (more) cur = nxt;
         }
-        if (more) cur = nxt;
-    }
 
-    if (G32) return;
+        if (G32) continue;
 
-    // ---- combine the K slices (fixed order) and store
-    if (ks > 1) {
-        float *mine = red + (size_t)wave * (R * 4 * 64);
-#pragma unroll
-        for (int rt = 0; rt < R; ++rt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) mine[(rt * 4 + r) * 64 + lane] = acc[rt][r];
-        __syncthreads();
-        if (kslice != 0) return;
-        for (int k2 = 1; k2 < ks; ++k2) {
-            const float *other = red + (size_t)(wave + k2) * (R * 4 * 64);
+        // ---- combine the K slices (fixed order; passes == 1 whenever ks > 1) and store
+        if (ks > 1) {
+            float *mine = red + (size_t)wave * (R * 4 * 64);
 #pragma unroll
             for (int rt = 0; rt < R; ++rt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[rt][r] += other[(rt * 4 + r) * 64 + lane];
+                for (int r = 0; r < 4; ++r) mine[(rt * 4 + r) * 64 + lane] = acc[rt][r];
+            __syncthreads();
+            if (kslice != 0) return;
+            for (int k2 = 1; k2 < ks; ++k2) {
+                const float *other = red + (size_t)(wave + k2) * (R * 4 * 64);
+#pragma unroll
+                for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[rt][r] += other[(rt * 4 + r) * 64 + lane];
+            }
         }
-    }
 #pragma unroll
-    for (int rt = 0; rt < R; ++rt) {
-        const int row = n0 + rt * 16 + op_row;
+        for (int rt = 0; rt < R; ++rt) {
+            const int row = n0 + rt * 16 + op_row;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int tok = 4 * kb + r;
-            if (row < N && tok < mt) {
-                const float y = acc[rt][r] / sdiv[r];
-                const size_t o = (size_t)(m0 + tok) * N + row;
-                if (a.out_f32)
-                    reinterpret_cast<float *>(a.out)[o] = y;
-                else
-                    reinterpret_cast<uint16_t *>(a.out)[o] = f32_to_bf16_rne(y);
+            for (int r = 0; r < 4; ++r) {
+                const int tok = 4 * kb + r;
+                if (row < N && tok < mt) {
+                    const float y = acc[rt][r] / sdiv[r];
+                    const size_t o = (size_t)(m0 + tok) * N + row;
+                    if (a.out_f32)
+                        reinterpret_cast<float *>(a.out)[o] = y;
+                    else
+                        reinterpret_cast<uint16_t *>(a.out)[o] = f32_to_bf16_rne(y);
+                }
+                acc[rt][r] = 0.0f;
             }
         }
     }
@@ -283,6 +310,8 @@ struct MfmaTuning {
     int min_width = 0;   // smallest M sent to this kernel; 0 = built-in default
     int row_tiles = 0;   // R: 1, 2 or 4; 0 = heuristic
     int k_split = 0;     // waves along K: 1, 2 or 4; 0 = heuristic
+    int passes = 0;      // row blocks per workgroup; 0 = heuristic
+    int engine = 0;      // 0 = choose, 1 = int8 MFMA only, 2 = FP4 x FP8 MFMA only
 };
 
 using MfmaKernelFn = void (*)(const MfmaArgs);
@@ -335,58 +364,11 @@ size_t mfma_lds_for(int ri, int mt, int K) {
                    : (ri == 1 ? mfma_lds_bytes<BITS, 2>(mt, K) : mfma_lds_bytes<BITS, 4>(mt, K));
 }
 
-// True when the MFMA kernel can take the shape: whole K tiles of four groups,
-// 16-byte aligned weight rows and 8-byte aligned scale rows.
+// True when the matrix-core kernels can take the shape: whole K tiles of four
+// groups, 16-byte aligned weight rows and 8-byte aligned scale rows.
 inline bool mfma_shape_ok(const void *B, const void *ws, int K) {
     return K % 512 == 0 && (reinterpret_cast<uintptr_t>(B) & 15) == 0 &&
            (ws == nullptr || (reinterpret_cast<uintptr_t>(ws) & 7) == 0);
-}
-
-// Launches the MFMA kernel; returns -1 when the shape does not fit in LDS (the
-// caller then uses the dot4 kernel), 0 on success, 2 on a launch error.
-template <int BITS>
-int launch_gemv_mfma(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
-                     int M, int N, int K, int out_kind, int scale_kind, int lds_limit,
-                     hipStream_t stream) {
-    const MfmaTuning &tu = mfma_tuning<BITS>();
-    const int ntok_tiles = (M + kMfmaTokens - 1) / kMfmaTokens;
-    const int mt = (M + ntok_tiles - 1) / ntok_tiles;
-
-    // Row tiles per wave and K split: enough workgroups to cover the chip a few
-    // times; long rows are split among the waves of a workgroup.
-    int ks = tu.k_split;
-    int R = tu.row_tiles;
-    const int ntiles = K / 512;
-    if (ks == 0) ks = (ntiles % 4 == 0 && (long)N * 4 <= 16384) ? 4 : ((ntiles % 2 == 0 && (long)N * 2 <= 16384) ? 2 : 1);
-    if (ks > ntiles) ks = 1;
-    if (R == 0) {
-        const long wgs1 = ((long)N + 16 * (4 / ks) - 1) / (16 * (4 / ks));  // workgroups at R = 1
-        R = wgs1 >= 8192 ? 4 : (wgs1 >= 2048 ? 2 : 1);
-    }
-    int ri = R == 4 ? 2 : (R == 2 ? 1 : 0);
-    while (ri > 0 && mfma_lds_for<BITS>(ri, mt, K) > (size_t)lds_limit) --ri;
-    if (mfma_lds_for<BITS>(ri, mt, K) > (size_t)lds_limit) return -1;
-    R = 1 << ri;
-
-    MfmaArgs args;
-    args.A = A;
-    args.B = B;
-    args.out = out;
-    args.s = s;
-    args.ws = reinterpret_cast<const uint16_t *>(ws);
-    args.M = M;
-    args.N = N;
-    args.K = K;
-    args.mt = mt;
-    args.ks_log2 = ks == 4 ? 2 : (ks == 2 ? 1 : 0);
-    args.out_f32 = out_kind == OUT_F32 ? 1 : 0;
-
-    const int rows_per_wg = 16 * R * (4 / ks);
-    const int grid_x = (N + rows_per_wg - 1) / rows_per_wg;
-    const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
-    hipLaunchKernelGGL(mfma_table<BITS>().fn[ri][variant], dim3(grid_x, ntok_tiles, 1),
-                       dim3(kMfmaThreads, 1, 1), mfma_lds_for<BITS>(ri, mt, K), stream, args);
-    return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
 }  // namespace bonsai

@@ -18,11 +18,13 @@ void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes) {
     t.passes = passes;
 }
 
-void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split) {
+void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine) {
     MfmaTuning &t = mfma_tuning<2>();
     t.min_width = min_width;
     t.row_tiles = row_tiles;
     t.k_split = k_split;
+    t.passes = passes;
+    t.engine = engine;
 }
 
 int t2g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,

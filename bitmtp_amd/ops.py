@@ -70,7 +70,7 @@ def load_t2_kernel() -> None:
     lib.t2g128_init.restype = ctypes.c_int
     lib.t2g128_set_tuning.argtypes = [ctypes.c_int] * 3
     lib.t2g128_set_tuning.restype = None
-    lib.t2g128_set_mfma_tuning.argtypes = [ctypes.c_int] * 3
+    lib.t2g128_set_mfma_tuning.argtypes = [ctypes.c_int] * 5
     lib.t2g128_set_mfma_tuning.restype = None
     _t2_lib = lib
 
@@ -92,7 +92,7 @@ def load_q1_kernel() -> None:
     lib.q1g128_init.restype = ctypes.c_int
     lib.q1g128_set_tuning.argtypes = [ctypes.c_int] * 3
     lib.q1g128_set_tuning.restype = None
-    lib.q1g128_set_mfma_tuning.argtypes = [ctypes.c_int] * 3
+    lib.q1g128_set_mfma_tuning.argtypes = [ctypes.c_int] * 5
     lib.q1g128_set_mfma_tuning.restype = None
     _q1_lib = lib
 

@@ -91,23 +91,28 @@ def test_launch_geometries(oracle, bits, lpr, waves, passes):
 
 
 @pytest.mark.parametrize("bits", [2, 1])
-@pytest.mark.parametrize("min_width,row_tiles,k_split", [
-    (1, 1, 1), (1, 2, 2), (1, 4, 4), (2, 1, 4), (2, 4, 1), (2, 2, 1), (1000, 0, 0),
+@pytest.mark.parametrize("engine", [1, 2])
+@pytest.mark.parametrize("min_width,row_tiles,k_split,passes", [
+    (1, 1, 1, 1), (1, 2, 2, 0), (1, 4, 4, 0), (2, 1, 4, 0), (2, 4, 1, 3), (2, 2, 1, 2),
+    (1, 1, 1, 5), (1000, 0, 0, 0),
 ])
-def test_mfma_geometries(oracle, bits, min_width, row_tiles, k_split):
-    """Matrix-core kernel: every row-tile / K-split combination, including a single
-    token sent through it, and the dot4 kernel forced for every width (1000)."""
+def test_mfma_geometries(oracle, bits, engine, min_width, row_tiles, k_split, passes):
+    """Both matrix-core kernels (1 = int8 MFMA, 2 = FP4 x FP8 MFMA): every row-tile /
+    K-split / pass combination, including a single token sent through them, and the
+    dot4 kernel forced for every width (min_width 1000)."""
     from bitmtp_amd import ops as O2
     lib = O2.t2_lib() if bits == 2 else O2.q1_lib()
     setter = lib.t2g128_set_mfma_tuning if bits == 2 else lib.q1g128_set_mfma_tuning
     try:
-        setter(min_width, row_tiles, k_split)
+        setter(min_width, row_tiles, k_split, passes, engine)
         for (M, N, K) in [(1, 70, 2048), (3, 257, 2560), (8, 50, 9728), (16, 33, 512),
                           (17, 130, 1024), (5, 16, 6144)]:
             p = oracle.synth_problem(min_width * 100 + row_tiles * 10 + k_split + K, M, N, K, bits)
-            check_problem(oracle, p, bits, f"mfma min={min_width} R={row_tiles} ks={k_split}")
+            check_problem(oracle, p, bits,
+                          f"mfma engine={engine} min={min_width} R={row_tiles} ks={k_split} "
+                          f"passes={passes}")
     finally:
-        setter(0, 0, 0)
+        setter(0, 0, 0, 0, 0)
 
 
 LAYER_17B = [(2048, 2048), (1024, 2048), (6144, 2048), (2048, 6144)]
