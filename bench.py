@@ -65,6 +65,21 @@ def make_pool(torch, n_layers: int, seed: int, dev):
     return pool
 
 
+def make_pool_matrix(torch, count: int, n: int, k: int, seed: int, dev):
+    """`count` distinct packed T2 matrices of one shape (same distributions as make_pool)."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    shifts = torch.tensor([1, 4, 16, 64], device=dev, dtype=torch.int32)
+    out = []
+    for _ in range(count):
+        codes = torch.randint(1, 4, (n, k // 4, 4), generator=gen, device=dev, dtype=torch.int32)
+        packed = (codes * shifts).sum(-1).to(torch.uint8).view(torch.int8).contiguous()
+        del codes
+        scales = torch.exp(torch.randn(n, k // 128, generator=gen, device=dev) * 0.5 - 4.0)
+        out.append((packed, scales.to(torch.bfloat16).contiguous()))
+    return out
+
+
 def make_activations(torch, ops, seed: int, dev):
     """fp16 N(0,1) activations per width and K, quantised per token on the GPU."""
     gen = torch.Generator(device=dev)
@@ -155,6 +170,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--layers", type=int, default=48, help="distinct layers in the weight pool")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--no-head", action="store_true", help="skip the lm_head-sized extra measurement")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device copy (for scaling rocprofv3 PMC byte counters)")
     args = ap.parse_args()
@@ -219,10 +235,35 @@ def main() -> int:
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "traffic": round(MEASURED_TRAFFIC_BYTES[dom]),
-        "kernel": f"gemv_dot4_kernel<BITS=2, MT={dom}, OUT=bf16> (width {dom})",
+        "kernel": (f"gemv_mfma_kernel<BITS=2> (width {dom})" if dom >= 5
+                   else f"gemv_dot4_kernel<BITS=2, MT={dom}> (width {dom})"),
         "bytes_per_launch": round(bytes_per_launch),
         "us_per_launch": per_width[dom]["us_per_launch"],
     }
+
+    # The one bandwidth-bound GEMV of the model, for scale: the packed lm_head
+    # (151936 x 2048, 82.7 MB) at the same widths, HBM-cold over a small pool.
+    head = {}
+    if not args.no_head:
+        hn, hk = 151936, 2048
+        hbytes = t2_bytes(hn, hk)
+        hpool = make_pool_matrix(torch, 8, hn, hk, seed=2, dev=dev)
+        hout = torch.empty(max(WIDTHS), hn, dtype=torch.bfloat16, device=dev)
+        for m in WIDTHS:
+            q, s_ = acts[(m, hk)]
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                spc = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for packed, scales in hpool:
+                    run.fn(q.data_ptr(), packed.data_ptr(), hout.data_ptr(), s_.data_ptr(),
+                           scales.data_ptr(), m, hn, hk, spc)
+            g.replay()
+            torch.cuda.synchronize()
+            t = min(run.time_graph(g) for _ in range(3)) / len(hpool)
+            head[str(m)] = {"us_per_launch": round(t * 1e6, 2), "gbps": round(hbytes / t / 1e9, 1),
+                            "pct_hbm_peak": round(hbytes / t / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+            del g
+        del hpool
 
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -245,6 +286,7 @@ def main() -> int:
             "pct_hbm_peak": round(gbps / HBM_PEAK_GBPS * 100, 2),
             "per_width": {str(m): per_width[m] for m in WIDTHS},
             "timing": "one HIP graph of all steps, HIP events on the launch stream, best of 3 replays",
+            "lm_head_151936x2048": head,
         },
         "roofline": roofline,
         "cpu_baseline": cpu,

@@ -1,9 +1,13 @@
 // Entry-point logic shared by libbonsai_t2.so and libbonsai_q1.so: argument
-// checks, one-time device set-up and the choice among the three kernels -- the
-// FP4 x FP8 matrix-core kernel (gemv_fp4.hip.h) whenever its staged activations
-// fit in LDS as one token tile, the int8 matrix-core kernel (gemv_mfma.hip.h)
-// for long rows at wide blocks, and the dot4 kernel (packed_gemv.hip.h) for
-// shapes neither takes (K not a multiple of 512, unaligned operands).  Replaces the if-chain over registered (M, N, K) of the
+// checks, one-time device set-up and the choice among the kernels.  Measured on
+// MI355X: the dot4 kernel (packed_gemv.hip.h) is fastest up to four tokens on
+// layer-sized matrices, the int8 matrix-core kernel (gemv_mfma.hip.h) from five
+// tokens on and from two tokens on for very long matrices (the lm_head).  The
+// FP4 x FP8 matrix-core kernel (gemv_fp4.hip.h) needs fewer VALU operations per
+// byte but its FP8 staging and deeper register use make it no faster yet; it
+// runs only when selected with the tuning call.  Shapes the matrix-core kernels
+// do not take (K not a multiple of 512, unaligned operands, token tiles that do
+// not fit in LDS) go to the dot4 kernel.  Replaces the if-chain over registered (M, N, K) of the
 // reference (src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:94-148).
 #ifndef BONSAI_GEMV_DISPATCH_HIP_H
 #define BONSAI_GEMV_DISPATCH_HIP_H
@@ -14,7 +18,8 @@
 
 namespace bonsai {
 
-constexpr int kDefaultMfmaMinWidth = 2;
+constexpr int kDefaultMfmaMinWidth = 5;       // layer-sized matrices
+constexpr int kLongMatrixRows = 32768;        // from here on the matrix cores pay off at M >= 2
 
 template <int BITS>
 int init_all_kernels() {
@@ -62,7 +67,7 @@ int launch_matrix_core(bool fp4, bool single_tile, const int8_t *A, const uint8_
         ks = (ntiles % 4 == 0 && (long)N * 4 <= 16384) ? 4
              : ((ntiles % 2 == 0 && (long)N * 2 <= 16384) ? 2 : 1);
     if (ks != 1 && ks != 2 && ks != 4) ks = 1;
-    if (ks > ntiles) ks = 1;
+    if (ks > ntiles || ntiles % ks != 0) ks = 1;  // equal K slices: the waves meet at one barrier
     if (R == 0) {
         const long wgs1 = ((long)N + 16 * (4 / ks) - 1) / (16 * (4 / ks));  // workgroups at R = 1
         R = wgs1 >= 8192 ? 4 : (wgs1 >= 2048 ? 2 : 1);
@@ -125,13 +130,14 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     const int lds_limit = st.lds_limit[dev];
 
     const MfmaTuning &mtu = mfma_tuning<BITS>();
-    const int min_width = mtu.min_width > 0 ? mtu.min_width : kDefaultMfmaMinWidth;
+    const int min_width = mtu.min_width > 0 ? mtu.min_width
+                                            : (N >= kLongMatrixRows ? 2 : kDefaultMfmaMinWidth);
     if (M >= min_width && mfma_shape_ok(B, out_kind == OUT_G32 ? nullptr : ws, K)) {
         int rc = -1;
-        if (mtu.engine != 1)
-            rc = launch_matrix_core<BITS>(true, mtu.engine == 0, A, B, out, s, ws, M, N, K, out_kind,
+        if (mtu.engine == 2)
+            rc = launch_matrix_core<BITS>(true, false, A, B, out, s, ws, M, N, K, out_kind,
                                           scale_kind, lds_limit, stream);
-        if (rc < 0 && mtu.engine != 2)
+        if (rc < 0)
             rc = launch_matrix_core<BITS>(false, false, A, B, out, s, ws, M, N, K, out_kind,
                                           scale_kind, lds_limit, stream);
         if (rc >= 0) return rc;

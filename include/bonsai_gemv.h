@@ -102,8 +102,8 @@ void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
 /* The same for the matrix-core kernels that serve widths >= min_width: smallest
  * width they take (a value above any M disables them), 16-row tiles per wave (1,
  * 2 or 4), waves of a workgroup splitting K (1, 2 or 4), row blocks a workgroup
- * walks through (used when K is not split) and the engine (1 = int8 MFMA only,
- * 2 = FP4 x FP8 MFMA only).  Zero = built-in choice. */
+ * walks through (used when K is not split) and the engine (2 = FP4 x FP8 MFMA,
+ * otherwise int8 MFMA).  Zero = built-in choice. */
 void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
 void q1g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
 
