@@ -105,6 +105,13 @@ def load_actq_kernel() -> None:
         ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
     ]
     lib.bonsai_act_quant_int8.restype = ctypes.c_int
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.bonsai_rmsnorm_quant_int8.argtypes = [vp, vp, ctypes.c_float, vp, vp, ci, ci, vp]
+    lib.bonsai_rmsnorm_quant_int8.restype = ci
+    lib.bonsai_add_rmsnorm_quant_int8.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, vp, ci, ci, vp]
+    lib.bonsai_add_rmsnorm_quant_int8.restype = ci
+    lib.bonsai_silu_mul_quant_int8.argtypes = [vp, vp, vp, ci, ci, vp]
+    lib.bonsai_silu_mul_quant_int8.restype = ci
     _actq_lib = lib
 
 
@@ -302,4 +309,69 @@ def quant_input(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
                                               _stream(x.device))
     if rc != 0:
         raise RuntimeError(f"quant_input: native launch failed with status {rc}")
+    return q, s
+
+
+def _check_bf16_rows(name: str, *tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t.dtype != torch.bfloat16 or not (t.is_cuda and t.is_contiguous()):
+            raise RuntimeError(f"{name}: operands must be contiguous CUDA bfloat16 tensors")
+
+
+def fused_norm_quant(x: torch.Tensor, w: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """RMSNorm then per-token INT8 quantisation: ``(q int8 [..., K], s fp32 [..., 1])``
+    (reference: ``_fused_norm_quant``, model.py:307-319)."""
+    _check_bf16_rows("fused_norm_quant", x, w)
+    k = x.shape[-1]
+    if w.shape != (k,) or k % 8 != 0:
+        raise RuntimeError("fused_norm_quant: weight must be [K] and K a multiple of 8")
+    m = x.numel() // k
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty(*x.shape[:-1], 1, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = actq_lib().bonsai_rmsnorm_quant_int8(_ptr(x), _ptr(w), float(eps), _ptr(q), _ptr(s), m, k,
+                                                  _stream(x.device))
+    if rc != 0:
+        raise RuntimeError(f"fused_norm_quant: native launch failed with status {rc}")
+    return q, s
+
+
+def fused_add_norm_quant(x: torch.Tensor, residual: torch.Tensor, w: torch.Tensor,
+                         eps: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``h = x + residual``; returns ``(h, q, s)`` with ``(q, s)`` the quantised RMSNorm of h
+    (reference: ``_fused_add_norm_quant``, model.py:322-336)."""
+    _check_bf16_rows("fused_add_norm_quant", x, residual, w)
+    k = x.shape[-1]
+    if residual.shape != x.shape or w.shape != (k,) or k % 8 != 0:
+        raise RuntimeError("fused_add_norm_quant: shape mismatch or K not a multiple of 8")
+    m = x.numel() // k
+    h = torch.empty_like(x)
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty(*x.shape[:-1], 1, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = actq_lib().bonsai_add_rmsnorm_quant_int8(_ptr(x), _ptr(residual), _ptr(w), float(eps),
+                                                      _ptr(h), _ptr(q), _ptr(s), m, k,
+                                                      _stream(x.device))
+    if rc != 0:
+        raise RuntimeError(f"fused_add_norm_quant: native launch failed with status {rc}")
+    return h, q, s
+
+
+def silu_mul_quant(gate_up: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``inner = silu(gate) * up`` of a merged gate/up projection ``[..., 2F]`` followed by
+    per-token quantisation: ``(q int8 [..., F], s fp32 [..., 1])`` (reference:
+    model.py:1058-1061)."""
+    _check_bf16_rows("silu_mul_quant", gate_up)
+    f2 = gate_up.shape[-1]
+    if f2 % 16 != 0:
+        raise RuntimeError("silu_mul_quant: last dimension must be 2F with F a multiple of 8")
+    f = f2 // 2
+    m = gate_up.numel() // f2
+    q = torch.empty(*gate_up.shape[:-1], f, dtype=torch.int8, device=gate_up.device)
+    s = torch.empty(*gate_up.shape[:-1], 1, dtype=torch.float32, device=gate_up.device)
+    with torch.cuda.device(gate_up.device):
+        rc = actq_lib().bonsai_silu_mul_quant_int8(_ptr(gate_up), _ptr(q), _ptr(s), m, f,
+                                                   _stream(gate_up.device))
+    if rc != 0:
+        raise RuntimeError(f"silu_mul_quant: native launch failed with status {rc}")
     return q, s

@@ -78,3 +78,19 @@ def unpack_q1_g128(packed: torch.Tensor) -> torch.Tensor:
     p = packed.view(torch.uint8).to(torch.int32)
     shifts = torch.arange(8, device=packed.device, dtype=torch.int32)
     return (2 * ((p.unsqueeze(-1) >> shifts) & 1) - 1).to(torch.int8).view(packed.shape[0], -1)
+
+
+def merge_packed_rows(parts):
+    """Concatenate packed projections that share their input along the output-row axis,
+    weights and group scales alike, so that one GEMV serves q/k/v or gate/up (reference:
+    ``prepare_merged_weights``, src/bonsai_sft/gpu/model.py:931-946,1042-1051).
+
+    ``parts`` is a sequence of ``(packed int8 [N_i, bytes], scales [N_i, K/128])``.
+    Returns ``(packed [sum N_i, bytes], scales [sum N_i, K/128], [N_i...])``."""
+    parts = list(parts)
+    cols = {p.shape[1] for p, _ in parts}
+    if len(cols) != 1:
+        raise ValueError("merged projections must share K")
+    packed = torch.cat([p for p, _ in parts], dim=0).contiguous()
+    scales = torch.cat([s for _, s in parts], dim=0).contiguous()
+    return packed, scales, [p.shape[0] for p, _ in parts]

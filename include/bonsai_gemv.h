@@ -120,6 +120,26 @@ void q1g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passe
 int bonsai_act_quant_int8(const void *x, int x_kind, int8_t *q, float *s, int M, int K,
                           void *stream);
 
+/* ---- fused producers of the GEMV input (libbonsai_actq.so) ------------------ */
+/* RMSNorm + per-token INT8 quantisation, the native form of `_fused_norm_quant`
+ * (src/bonsai_sft/gpu/model.py:307-319): x, w bf16; q int8 [M,K]; s fp32 [M].
+ *   var = mean(fp32(x)^2); normed = bf16(w * bf16(fp32(x) * rsqrt(var + eps)));
+ *   (q, s) = quantisation of fp32(normed) as in bonsai_act_quant_int8. */
+int bonsai_rmsnorm_quant_int8(const void *x, const void *w, float eps, int8_t *q, float *s, int M,
+                              int K, void *stream);
+
+/* Residual add + RMSNorm + quantisation, `_fused_add_norm_quant`
+ * (src/bonsai_sft/gpu/model.py:322-336): h_out = bf16(x + residual) [M,K] is also
+ * returned, then as above on h_out. */
+int bonsai_add_rmsnorm_quant_int8(const void *x, const void *residual, const void *w, float eps,
+                                  void *h_out, int8_t *q, float *s, int M, int K, void *stream);
+
+/* SiLU(gate) * up + quantisation of the merged gate/up GEMV output
+ * (src/bonsai_sft/gpu/model.py:1058-1061): gate_up bf16 [M, 2F] with the gate in
+ * columns [0,F) and up in [F,2F); inner = bf16(bf16(silu(gate)) * up); q int8
+ * [M,F], s fp32 [M]. */
+int bonsai_silu_mul_quant_int8(const void *gate_up, int8_t *q, float *s, int M, int F, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

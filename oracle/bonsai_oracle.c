@@ -260,4 +260,96 @@ void oracle_gemv(const int8_t *A, const uint8_t *B, const float *S, const uint16
     }
 }
 
-int oracle_abi_version(void) { return 1; }
+/* ---- fused norm / activation producers (model.py:307-336, 1058-1061) ---- */
+
+static inline float bf16_round_f(float f) { return oracle_bf16_to_f32(oracle_f32_to_bf16(f)); }
+
+/* Sum of fp32 squares in fp64, in the order the HIP kernel uses: 256 threads, thread t
+ * takes the 8-element vectors t, t+256, ... in turn; xor butterfly (32,16,..,1) inside
+ * each 64-thread wave; the four wave totals added left to right. */
+static double sumsq_kernel_order(const float *h, int K) {
+    double lane[256];
+    int nvec = K / 8;
+    for (int t = 0; t < 256; ++t) {
+        double acc = 0.0;
+        for (int v = t; v < nvec; v += 256)
+            for (int i = 0; i < 8; ++i) {
+                volatile float sq = h[8 * v + i] * h[8 * v + i];
+                acc += (double)sq;
+            }
+        lane[t] = acc;
+    }
+    double total = 0.0;
+    for (int w = 0; w < 4; ++w) {
+        double a[64], b[64];
+        for (int i = 0; i < 64; ++i) a[i] = lane[64 * w + i];
+        for (int off = 32; off > 0; off >>= 1) {
+            for (int i = 0; i < 64; ++i) b[i] = a[i] + a[i ^ off];
+            for (int i = 0; i < 64; ++i) a[i] = b[i];
+        }
+        total = (w == 0) ? a[0] : total + a[0];
+    }
+    return total;
+}
+
+static void quant_row(const float *nf, int8_t *q, float *s, int K) {
+    float amax = 0.0f;
+    for (int k = 0; k < K; ++k) {
+        float a = fabsf(nf[k]);
+        if (a > amax) amax = a;
+    }
+    if (amax < 1e-5f) amax = 1e-5f;
+    volatile float recip = 1.0f / amax;
+    float sv = recip * 127.0f;
+    *s = sv;
+    for (int k = 0; k < K; ++k) {
+        float r = rintf(nf[k] * sv);
+        if (r < -128.0f) r = -128.0f;
+        if (r > 127.0f) r = 127.0f;
+        q[k] = (int8_t)r;
+    }
+}
+
+/* _fused_norm_quant / _fused_add_norm_quant.  X, RES (may be NULL), W are bf16 bit
+ * patterns; H (may be NULL) receives bf16(x + residual).  K <= 65536. */
+void oracle_rmsnorm_quant(const uint16_t *X, const uint16_t *RES, const uint16_t *W, float eps,
+                          uint16_t *H, int8_t *Q, float *S, int M, int K) {
+    static float h[65536], nf[65536];
+    for (int m = 0; m < M; ++m) {
+        for (int k = 0; k < K; ++k) {
+            float v = oracle_bf16_to_f32(X[(size_t)m * K + k]);
+            if (RES) {
+                volatile float sum = v + oracle_bf16_to_f32(RES[(size_t)m * K + k]);
+                v = bf16_round_f(sum);
+                if (H) H[(size_t)m * K + k] = oracle_f32_to_bf16(v);
+            }
+            h[k] = v;
+        }
+        float var = (float)sumsq_kernel_order(h, K) / (float)K;
+        volatile float root = sqrtf(var + eps);
+        float rs = 1.0f / root;
+        for (int k = 0; k < K; ++k) {
+            volatile float t = h[k] * rs;
+            volatile float u = oracle_bf16_to_f32(W[k]) * bf16_round_f(t);
+            nf[k] = bf16_round_f(u);
+        }
+        quant_row(nf, Q + (size_t)m * K, S + m, K);
+    }
+}
+
+/* SiLU(gate) * up + quant: GU bf16 [M, 2F]; inner = bf16(bf16(g / (1 + exp(-g))) * u). */
+void oracle_silu_mul_quant(const uint16_t *GU, int8_t *Q, float *S, int M, int F) {
+    static float nf[65536];
+    for (int m = 0; m < M; ++m) {
+        const uint16_t *g = GU + (size_t)m * 2 * F, *u = g + F;
+        for (int k = 0; k < F; ++k) {
+            float gv = oracle_bf16_to_f32(g[k]);
+            volatile float sg = gv / (1.0f + expf(-gv));
+            volatile float pr = bf16_round_f(sg) * oracle_bf16_to_f32(u[k]);
+            nf[k] = bf16_round_f(pr);
+        }
+        quant_row(nf, Q + (size_t)m * F, S + m, F);
+    }
+}
+
+int oracle_abi_version(void) { return 2; }

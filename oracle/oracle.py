@@ -53,6 +53,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_act_quant.argtypes = [vp, vp, vp, ci, ci]
         L.oracle_group_sums.argtypes = [vp, vp, vp, ci, ci, ci, ci]
         L.oracle_gemv.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
+        L.oracle_rmsnorm_quant.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, vp, ci, ci]
+        L.oracle_rmsnorm_quant.restype = None
+        L.oracle_silu_mul_quant.argtypes = [vp, vp, vp, ci, ci]
+        L.oracle_silu_mul_quant.restype = None
         L.oracle_f32_to_bf16.argtypes = [ctypes.c_float]
         L.oracle_f32_to_bf16.restype = ctypes.c_uint16
         L.oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
@@ -126,6 +130,32 @@ def c_act_quant(X: np.ndarray):
     Q = np.empty((M, K), dtype=np.int8)
     S = np.empty((M,), dtype=np.float32)
     lib().oracle_act_quant(_p(X), _p(Q), _p(S), M, K)
+    return Q, S
+
+
+def c_rmsnorm_quant(x_bits, w_bits, eps: float, residual_bits=None):
+    """bf16 bit patterns in; returns (q int8 [M,K], s fp32 [M], h bf16 bits or None)."""
+    X = _c(x_bits, np.uint16)
+    W = _c(w_bits, np.uint16)
+    M, K = X.shape
+    Q = np.empty((M, K), dtype=np.int8)
+    S = np.empty((M,), dtype=np.float32)
+    if residual_bits is None:
+        lib().oracle_rmsnorm_quant(_p(X), None, _p(W), eps, None, _p(Q), _p(S), M, K)
+        return Q, S, None
+    R = _c(residual_bits, np.uint16)
+    H = np.empty((M, K), dtype=np.uint16)
+    lib().oracle_rmsnorm_quant(_p(X), _p(R), _p(W), eps, _p(H), _p(Q), _p(S), M, K)
+    return Q, S, H
+
+
+def c_silu_mul_quant(gu_bits):
+    GU = _c(gu_bits, np.uint16)
+    M, F2 = GU.shape
+    F = F2 // 2
+    Q = np.empty((M, F), dtype=np.int8)
+    S = np.empty((M,), dtype=np.float32)
+    lib().oracle_silu_mul_quant(_p(GU), _p(Q), _p(S), M, F)
     return Q, S
 
 
