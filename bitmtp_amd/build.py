@@ -24,6 +24,7 @@ TARGETS = {
     "t2g128_kernels.hip": os.path.join("t2g128_kernels", "libbonsai_t2.so"),
     "q1g128_kernels.hip": os.path.join("q1g128_kernels", "libbonsai_q1.so"),
     "act_quant.hip": os.path.join("act_quant", "libbonsai_actq.so"),
+    "decode_ops.hip": os.path.join("decode_ops", "libbonsai_decode.so"),
 }
 
 HIPCC_FLAGS = [
@@ -42,7 +43,8 @@ def lib_path(source: str) -> str:
 
 def _deps() -> list[str]:
     return [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [
-        os.path.join(HERE, "..", "include", "bonsai_gemv.h")]
+        os.path.join(HERE, "..", "include", "bonsai_gemv.h"),
+        os.path.join(HERE, "..", "include", "bonsai_decode.h")]
 
 
 def _stale(out: str) -> bool:

@@ -1,0 +1,580 @@
+// libbonsai_decode.so: the ops between the packed GEMVs of one decode step on gfx950.
+//
+//   qk_norm_rope_kernel   split + per-head q/k RMSNorm + RoPE + KV write
+//                         (src/bonsai_sft/gpu/model.py:388-436)
+//   attn_partial_kernel   softmax(q k^T) v over one 64-slot chunk of the shared KV
+//   attn_combine_kernel   merges the chunks, rounds to bf16 and quantises per token
+//                         (src/bonsai_sft/gpu/model.py:996-1005)
+//   kv_commit_kernel      workspace rows -> history rows (fast_runtime.py:467-508)
+//   draft_rows_kernel / draft_accept_kernel   argmax + confidence chain
+//                         (src/bonsai_sft/gpu/fast_generate.py:111-130)
+//
+// Attention is HBM/L2-bound integer-free fp work: per layer it reads
+// 2 * n_kv * (cache_len + M) * 256 bytes of KV once per query-head group.  The mask
+// is not a tensor: history visibility is `slot < cache_len && slot != hide`, workspace
+// visibility one 32-bit word per row, both read from a small device descriptor, so a
+// replayed graph only touches the live part of the buffer.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/bonsai_decode.h"
+
+namespace {
+
+constexpr int kHd = BONSAI_HEAD_DIM;
+constexpr int kChunk = BONSAI_ATTN_CHUNK;
+constexpr int kPartStride = kHd + 4;  // 128 accumulators + running max + running sum, 16-byte pitch
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ float bf16_round(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    bf16x2_t x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    return __builtin_amdgcn_fdot2_f32_bf16(x, y, c, false);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// q/k RMSNorm + RoPE + KV write.  One wave per (token, head); lane i holds the
+// element pair (i, i + 64), which is the pair rotate_half exchanges.
+// The sum of squares is accumulated in fp64 (lane pair, then an xor butterfly), so
+// its fp32 value does not depend on the summation order to within one rounding.
+// ---------------------------------------------------------------------------
+struct RopeArgs {
+    const uint16_t *xqkv;
+    const uint16_t *qw;
+    const uint16_t *kw;
+    const uint16_t *cos_t;
+    const uint16_t *sin_t;
+    const int32_t *positions;
+    uint16_t *q_out;
+    uint16_t *k_layer;
+    uint16_t *v_layer;
+    float eps;
+    int M, n_heads, n_kv, slots, write_slot, max_pos;
+};
+
+__global__ void __launch_bounds__(256) qk_norm_rope_kernel(RopeArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int m = blockIdx.y;
+    const int total_heads = a.n_heads + 2 * a.n_kv;
+    if (head >= total_heads) return;
+    const uint16_t *x = a.xqkv + ((size_t)m * total_heads + head) * kHd;
+    const uint32_t r0 = x[lane], r1 = x[lane + 64];
+
+    if (head >= a.n_heads + a.n_kv) {  // V: plain copy into the workspace row
+        const int vh = head - a.n_heads - a.n_kv;
+        uint16_t *dst = a.v_layer + ((size_t)vh * a.slots + a.write_slot + m) * kHd;
+        dst[lane] = (uint16_t)r0;
+        dst[lane + 64] = (uint16_t)r1;
+        return;
+    }
+    const bool is_q = head < a.n_heads;
+    const uint16_t *w = is_q ? a.qw : a.kw;
+    const float f0 = bf16_bits_to_f32(r0), f1 = bf16_bits_to_f32(r1);
+    double ss = (double)(f0 * f0) + (double)(f1 * f1);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    const float var = (float)ss / (float)kHd;
+    const float rs = 1.0f / sqrtf(var + a.eps);
+    const float n0 = bf16_round(bf16_bits_to_f32(w[lane]) * bf16_round(f0 * rs));
+    const float n1 = bf16_round(bf16_bits_to_f32(w[lane + 64]) * bf16_round(f1 * rs));
+
+    int pos = a.positions[m];
+    pos = pos < 0 ? 0 : (pos >= a.max_pos ? a.max_pos - 1 : pos);
+    const uint16_t *cr = a.cos_t + (size_t)pos * kHd;
+    const uint16_t *sr = a.sin_t + (size_t)pos * kHd;
+    const float c0 = bf16_bits_to_f32(cr[lane]), c1 = bf16_bits_to_f32(cr[lane + 64]);
+    const float s0 = bf16_bits_to_f32(sr[lane]), s1 = bf16_bits_to_f32(sr[lane + 64]);
+    // rotate_half(n) = [-n_hi, n_lo]
+    const float o0 = bf16_round(bf16_round(n0 * c0) + bf16_round(-n1 * s0));
+    const float o1 = bf16_round(bf16_round(n1 * c1) + bf16_round(n0 * s1));
+
+    uint16_t *dst = is_q ? a.q_out + ((size_t)m * a.n_heads + head) * kHd
+                         : a.k_layer + ((size_t)(head - a.n_heads) * a.slots + a.write_slot + m) * kHd;
+    dst[lane] = (uint16_t)f32_to_bf16_bits(o0);
+    dst[lane + 64] = (uint16_t)f32_to_bf16_bits(o1);
+}
+
+// ---------------------------------------------------------------------------
+// Attention, split over KV chunks.  One wave per (kv head, query head of the group,
+// chunk, row group of RW rows).  Logical sequence index t in [0, cache_len + M):
+// t < cache_len is history slot t, otherwise workspace slot sigma + (t - cache_len).
+//   phase 1 (lane = slot):  the lane keeps its K row (64 dwords) in registers; the q
+//                           row is wave-uniform; s = scale * <q, k> with v_dot2_f32_bf16
+//   softmax statistics of the chunk per row (wave reductions), p parked in LDS
+//   phase 2 (lane = 2 dims): acc[r] += p[r][slot] * V[slot][dims], V rows read
+//                           coalesced (256 B per slot)
+// Partials: [M][n_heads][n_chunks][132] fp32 = 128 unnormalised sums, max, sum, 2 unused.
+// The workgroup id puts the kv head in the low three bits, so with 8 kv heads all
+// waves that share a kv head run on one XCD and share its L2.
+// ---------------------------------------------------------------------------
+struct AttnArgs {
+    const uint32_t *q;        // [M][n_heads][64] bf16 pairs
+    const uint32_t *k_layer;  // [n_kv][slots][64]
+    const uint32_t *v_layer;
+    const int32_t *meta;
+    float *part;
+    float scale_log2e;        // scale * log2(e): softmax runs in base 2
+    int M, n_heads, n_kv, hpg, slots, sigma, n_chunks, row_groups;
+};
+
+template <int RW>
+__global__ void __launch_bounds__(64) attn_partial_kernel(AttnArgs a) {
+    __shared__ float p_lds[RW][kChunk];
+    const int lane = threadIdx.x;
+    int id = blockIdx.x;
+    const int kvh = id % a.n_kv;
+    id /= a.n_kv;
+    const int chunk = id % a.n_chunks;
+    id /= a.n_chunks;
+    const int g = id % a.hpg;
+    const int rg = id / a.hpg;
+    const int head = kvh * a.hpg + g;
+
+    // a descriptor that does not fit the segment is clamped, never followed out of bounds
+    const int cache_len = min(max(a.meta[0], 0), a.sigma);
+    const int hide = a.meta[1];
+    const int total = cache_len + a.M;
+    const int t0 = chunk * kChunk;
+    if (t0 >= total) return;  // nothing live in this chunk; the combine step skips it too
+    const int n_live = min(kChunk, total - t0);
+
+    // ---- phase 1: scores of this lane's slot against RW rows
+    const int t = t0 + lane;
+    const bool live = lane < n_live;
+    const int tc = live ? t : t0;  // clamped: dead lanes read a valid row and are masked
+    const int slot = tc < cache_len ? tc : a.sigma + (tc - cache_len);
+    const uint4 *krow = reinterpret_cast<const uint4 *>(a.k_layer + ((size_t)kvh * a.slots + slot) * 64);
+    uint4 kreg[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) kreg[i] = krow[i];
+
+    const int row0 = rg * RW;
+    float mrow[RW], lrow[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        const int m = min(row0 + r, a.M - 1);
+        const uint4 *qrow = reinterpret_cast<const uint4 *>(a.q + ((size_t)m * a.n_heads + head) * 64);
+        float acc0 = 0.0f, acc1 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint4 qv = qrow[i];  // wave-uniform address
+            acc0 = dot2_bf16(kreg[i].x, qv.x, acc0);
+            acc1 = dot2_bf16(kreg[i].y, qv.y, acc1);
+            acc0 = dot2_bf16(kreg[i].z, qv.z, acc0);
+            acc1 = dot2_bf16(kreg[i].w, qv.w, acc1);
+        }
+        bool vis = live;
+        if (t < cache_len) {
+            vis = vis && (t != hide);
+        } else {
+            const uint32_t wmask = (uint32_t)a.meta[2 + m];
+            vis = vis && ((wmask >> ((t - cache_len) & 31)) & 1u);
+        }
+        const float sc = vis ? (acc0 + acc1) * a.scale_log2e : -INFINITY;
+        const float mx = wave_max(sc);
+        const float p = (mx == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(sc - mx);
+        mrow[r] = mx;
+        lrow[r] = wave_sum(p);
+        p_lds[r][lane] = p;
+    }
+    __syncthreads();
+
+    // ---- phase 2: acc[r][2 dims] over the live slots of the chunk
+    float acc[RW][2];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) acc[r][0] = acc[r][1] = 0.0f;
+    const uint32_t *vbase = a.v_layer + (size_t)kvh * a.slots * 64 + lane;
+    constexpr int UN = 8;
+    for (int j0 = 0; j0 < n_live; j0 += UN) {
+        uint32_t vv[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int tj = min(t0 + j0 + u, total - 1);
+            const int sj = tj < cache_len ? tj : a.sigma + (tj - cache_len);
+            vv[u] = vbase[(size_t)sj * 64];
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const float v0 = bf16_bits_to_f32(vv[u] & 0xffffu);
+            const float v1 = __uint_as_float(vv[u] & 0xffff0000u);
+            const bool in = (j0 + u) < n_live;
+#pragma unroll
+            for (int r = 0; r < RW; ++r) {
+                const float p = in ? p_lds[r][j0 + u] : 0.0f;
+                acc[r][0] = fmaf(p, v0, acc[r][0]);
+                acc[r][1] = fmaf(p, v1, acc[r][1]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        const int m = row0 + r;
+        if (m < a.M) {
+            float *dst = a.part + (((size_t)m * a.n_heads + head) * a.n_chunks + chunk) * kPartStride;
+            reinterpret_cast<float2 *>(dst)[lane] = make_float2(acc[r][0], acc[r][1]);
+            if (lane == 0) {
+                dst[kHd] = mrow[r];
+                dst[kHd + 1] = lrow[r];
+            }
+        }
+    }
+}
+
+// One workgroup per token: merge the chunk partials of every head, round to bf16,
+// then quantise the whole row (all heads) per token like `quant_input`.
+struct CombineArgs {
+    const float *part;
+    const int32_t *meta;
+    uint16_t *out_bf16;
+    int8_t *out_q;
+    float *out_s;
+    int M, n_heads, n_chunks, sigma;
+};
+
+constexpr int kCombineThreads = 256;
+constexpr int kCombineMaxVec = 2;  // 8-element vectors per thread: up to 32 heads
+
+__global__ void __launch_bounds__(kCombineThreads) attn_combine_kernel(CombineArgs a) {
+    __shared__ float max_scratch[kCombineThreads / 64];
+    const int m = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int total = min(max(a.meta[0], 0), a.sigma) + a.M;
+    const int live_chunks = (total + kChunk - 1) / kChunk;
+    const int nvec = a.n_heads * (kHd / 8);
+    float o[kCombineMaxVec][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int it = 0; it < kCombineMaxVec; ++it) {
+        const int v = tid + it * kCombineThreads;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[it][i] = 0.0f;
+        if (v >= nvec) continue;
+        const int head = v / (kHd / 8);
+        const int d0 = (v % (kHd / 8)) * 8;
+        const float *base = a.part + ((size_t)m * a.n_heads + head) * a.n_chunks * kPartStride;
+        float mx = -INFINITY;
+        for (int c = 0; c < live_chunks; ++c) mx = fmaxf(mx, base[(size_t)c * kPartStride + kHd]);
+        float den = 0.0f;
+        float num[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) num[i] = 0.0f;
+        if (mx != -INFINITY) {
+            for (int c = 0; c < live_chunks; ++c) {
+                const float *pc = base + (size_t)c * kPartStride;
+                const float mc = pc[kHd];
+                if (mc == -INFINITY) continue;
+                const float wgt = __builtin_amdgcn_exp2f(mc - mx);
+                den = fmaf(wgt, pc[kHd + 1], den);
+                const float4 x0 = reinterpret_cast<const float4 *>(pc + d0)[0];
+                const float4 x1 = reinterpret_cast<const float4 *>(pc + d0)[1];
+                num[0] = fmaf(wgt, x0.x, num[0]); num[1] = fmaf(wgt, x0.y, num[1]);
+                num[2] = fmaf(wgt, x0.z, num[2]); num[3] = fmaf(wgt, x0.w, num[3]);
+                num[4] = fmaf(wgt, x1.x, num[4]); num[5] = fmaf(wgt, x1.y, num[5]);
+                num[6] = fmaf(wgt, x1.z, num[6]); num[7] = fmaf(wgt, x1.w, num[7]);
+            }
+        }
+        const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            o[it][i] = bf16_round(num[i] * inv);
+            amax = fmaxf(amax, fabsf(o[it][i]));
+        }
+        if (a.out_bf16 != nullptr) {
+            uint4 w;
+            w.x = f32_to_bf16_bits(o[it][0]) | (f32_to_bf16_bits(o[it][1]) << 16);
+            w.y = f32_to_bf16_bits(o[it][2]) | (f32_to_bf16_bits(o[it][3]) << 16);
+            w.z = f32_to_bf16_bits(o[it][4]) | (f32_to_bf16_bits(o[it][5]) << 16);
+            w.w = f32_to_bf16_bits(o[it][6]) | (f32_to_bf16_bits(o[it][7]) << 16);
+            reinterpret_cast<uint4 *>(a.out_bf16 + (size_t)m * nvec * 8)[v] = w;
+        }
+    }
+    if (a.out_q == nullptr) return;  // uniform over the grid
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) max_scratch[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(max_scratch[0], max_scratch[1]), fmaxf(max_scratch[2], max_scratch[3]));
+    const float sval = (1.0f / fmaxf(amax, 1e-5f)) * 127.0f;
+    if (tid == 0) a.out_s[m] = sval;
+#pragma unroll
+    for (int it = 0; it < kCombineMaxVec; ++it) {
+        const int v = tid + it * kCombineThreads;
+        if (v >= nvec) continue;
+        uint32_t b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float r = __builtin_rintf(o[it][i] * sval);
+            r = fminf(fmaxf(r, -128.0f), 127.0f);
+            b[i] = (uint32_t)((int)r) & 0xffu;
+        }
+        uint2 w;
+        w.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        w.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+        reinterpret_cast<uint2 *>(a.out_q + (size_t)m * nvec * 8)[v] = w;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// KV commit: rows [src, src+n) -> [dst, dst+n) for every (k|v, layer, kv head).
+// One thread per 16 bytes.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) kv_commit_kernel(uint4 *kv, int planes, int slots, int src,
+                                                        int dst, int n) {
+    const int per_plane = n * (kHd * 2 / 16);
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= planes * per_plane) return;
+    const int plane = idx / per_plane;
+    const int off = idx % per_plane;
+    uint4 *base = kv + (size_t)plane * slots * (kHd * 2 / 16);
+    base[(size_t)dst * (kHd * 2 / 16) + off] = base[(size_t)src * (kHd * 2 / 16) + off];
+}
+
+// ---------------------------------------------------------------------------
+// Draft chain.  One workgroup of 1024 threads per logits row: running (max, index)
+// and the sum of exp(x - max) in one pass with 16-byte loads; conf = 1 / sum.
+// ---------------------------------------------------------------------------
+constexpr int kDraftThreads = 1024;
+
+struct RowStat {
+    float mx;
+    int idx;
+    float sum;
+};
+
+__device__ __forceinline__ RowStat merge(RowStat a, RowStat b) {
+    // larger max wins; equal maxima keep the lower index
+    const bool take_b = (b.mx > a.mx) || (b.mx == a.mx && b.idx < a.idx);
+    const float mx = fmaxf(a.mx, b.mx);
+    RowStat r;
+    r.mx = mx;
+    r.idx = take_b ? b.idx : a.idx;
+    const float sa = (a.mx == -INFINITY) ? 0.0f : a.sum * __builtin_amdgcn_exp2f((a.mx - mx) * 1.44269504f);
+    const float sb = (b.mx == -INFINITY) ? 0.0f : b.sum * __builtin_amdgcn_exp2f((b.mx - mx) * 1.44269504f);
+    r.sum = sa + sb;
+    return r;
+}
+
+__global__ void __launch_bounds__(kDraftThreads)
+draft_rows_kernel(const uint16_t *logits, int ld, int vocab, int32_t *tokens, float *conf) {
+    __shared__ RowStat wave_stat[kDraftThreads / 64];
+    const int row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const uint16_t *x = logits + (size_t)row * ld;
+    RowStat st;
+    st.mx = -INFINITY;
+    st.idx = 0x7fffffff;
+    st.sum = 0.0f;
+    const int nvec = vocab / 8;
+    for (int v = tid; v < nvec; v += kDraftThreads) {
+        const uint4 raw = reinterpret_cast<const uint4 *>(x)[v];
+        const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+        float e[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            e[2 * i] = bf16_bits_to_f32(d[i] & 0xffffu);
+            e[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+        }
+        float vm = e[0];
+        int vi = 0;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+            if (e[i] > vm) {
+                vm = e[i];
+                vi = i;
+            }
+        }
+        if (!(vm == vm)) continue;  // a NaN vector contributes nothing
+        const float nm = fmaxf(st.mx, vm);
+        float s = (st.mx == -INFINITY) ? 0.0f : st.sum * __builtin_amdgcn_exp2f((st.mx - nm) * 1.44269504f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += __builtin_amdgcn_exp2f((e[i] - nm) * 1.44269504f);
+        if (vm > st.mx) st.idx = v * 8 + vi;
+        st.mx = nm;
+        st.sum = s;
+    }
+    for (int c = nvec * 8 + tid; c < vocab; c += kDraftThreads) {  // ragged tail
+        RowStat one;
+        one.mx = bf16_bits_to_f32(x[c]);
+        one.idx = c;
+        one.sum = 1.0f;
+        if (one.mx == one.mx) st = merge(st, one);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        RowStat o;
+        o.mx = __shfl_xor(st.mx, off);
+        o.idx = __shfl_xor(st.idx, off);
+        o.sum = __shfl_xor(st.sum, off);
+        st = merge(st, o);
+    }
+    if ((tid & 63) == 0) wave_stat[tid >> 6] = st;
+    __syncthreads();
+    if (tid == 0) {
+        RowStat t = wave_stat[0];
+        for (int w = 1; w < kDraftThreads / 64; ++w) t = merge(t, wave_stat[w]);
+        tokens[row] = t.idx == 0x7fffffff ? 0 : t.idx;
+        conf[row] = t.sum > 0.0f ? 1.0f / t.sum : 0.0f;
+    }
+}
+
+__global__ void draft_accept_kernel(const float *conf, int rows, float threshold, int32_t *accept) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int n = 1;
+    for (int r = 1; r < rows; ++r) {
+        if (!(conf[r] > threshold)) break;
+        ++n;
+    }
+    accept[0] = n;
+    accept[1] = rows;
+}
+
+int rows_per_wave(int M) {
+    // few rows per wave keep phase 2 short; more row groups re-read K/V from L2
+    if (M <= 4) return M;
+    if (M <= 12) return 3;
+    return 4;
+}
+
+}  // namespace
+
+extern "C" int bonsai_qk_norm_rope_kv_write(const void *xqkv, const void *q_norm_w,
+                                            const void *k_norm_w, float eps, const void *cos_table,
+                                            const void *sin_table, const int32_t *positions,
+                                            void *q_out, void *k_layer, void *v_layer, int M,
+                                            int n_heads, int n_kv, int slots, int write_slot,
+                                            int max_pos, void *stream) {
+    if (!xqkv || !q_norm_w || !k_norm_w || !cos_table || !sin_table || !positions || !q_out ||
+        !k_layer || !v_layer)
+        return BONSAI_DECODE_ERR_ARG;
+    if (M < 1 || M > BONSAI_MAX_WIDTH || n_heads < 1 || n_kv < 1 || max_pos < 1 || write_slot < 0 ||
+        write_slot + M > slots)
+        return BONSAI_DECODE_ERR_ARG;
+    RopeArgs a;
+    a.xqkv = static_cast<const uint16_t *>(xqkv);
+    a.qw = static_cast<const uint16_t *>(q_norm_w);
+    a.kw = static_cast<const uint16_t *>(k_norm_w);
+    a.cos_t = static_cast<const uint16_t *>(cos_table);
+    a.sin_t = static_cast<const uint16_t *>(sin_table);
+    a.positions = positions;
+    a.q_out = static_cast<uint16_t *>(q_out);
+    a.k_layer = static_cast<uint16_t *>(k_layer);
+    a.v_layer = static_cast<uint16_t *>(v_layer);
+    a.eps = eps;
+    a.M = M;
+    a.n_heads = n_heads;
+    a.n_kv = n_kv;
+    a.slots = slots;
+    a.write_slot = write_slot;
+    a.max_pos = max_pos;
+    const int total_heads = n_heads + 2 * n_kv;
+    hipLaunchKernelGGL(qk_norm_rope_kernel, dim3((total_heads + 3) / 4, M), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a);
+    return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int slots) {
+    if (M < 1 || n_heads < 1 || slots < 1) return 0;
+    const int64_t n_chunks = (slots + kChunk - 1) / kChunk;
+    return (int64_t)M * n_heads * n_chunks * kPartStride * (int64_t)sizeof(float);
+}
+
+extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const void *v_layer,
+                                       const int32_t *meta, void *scratch, void *out_bf16,
+                                       int8_t *out_q, float *out_s, float scale, int M, int n_heads,
+                                       int n_kv, int slots, int sigma, void *stream) {
+    if (!q || !k_layer || !v_layer || !meta || !scratch) return BONSAI_DECODE_ERR_ARG;
+    if ((out_q == nullptr) != (out_s == nullptr)) return BONSAI_DECODE_ERR_ARG;
+    if (!out_bf16 && !out_q) return BONSAI_DECODE_ERR_ARG;
+    if (M < 1 || M > BONSAI_MAX_WIDTH || n_kv < 1 || n_heads < n_kv || n_heads % n_kv != 0 ||
+        n_heads > kCombineThreads * kCombineMaxVec / (kHd / 8) || sigma < 0 || sigma + M > slots)
+        return BONSAI_DECODE_ERR_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    AttnArgs a;
+    a.q = static_cast<const uint32_t *>(q);
+    a.k_layer = static_cast<const uint32_t *>(k_layer);
+    a.v_layer = static_cast<const uint32_t *>(v_layer);
+    a.meta = meta;
+    a.part = static_cast<float *>(scratch);
+    a.scale_log2e = scale * 1.44269504088896340736f;
+    a.M = M;
+    a.n_heads = n_heads;
+    a.n_kv = n_kv;
+    a.hpg = n_heads / n_kv;
+    a.slots = slots;
+    a.sigma = sigma;
+    // the live length is cache_len + M <= sigma + M: chunks beyond it are never launched
+    a.n_chunks = (sigma + M + kChunk - 1) / kChunk;
+    const int rw = rows_per_wave(M);
+    a.row_groups = (M + rw - 1) / rw;
+    const AttnArgs &launch = a;
+    const int blocks = n_kv * a.n_chunks * a.hpg * a.row_groups;
+    switch (rw) {
+        case 1: hipLaunchKernelGGL(attn_partial_kernel<1>, dim3(blocks), dim3(64), 0, st, launch); break;
+        case 2: hipLaunchKernelGGL(attn_partial_kernel<2>, dim3(blocks), dim3(64), 0, st, launch); break;
+        case 3: hipLaunchKernelGGL(attn_partial_kernel<3>, dim3(blocks), dim3(64), 0, st, launch); break;
+        default: hipLaunchKernelGGL(attn_partial_kernel<4>, dim3(blocks), dim3(64), 0, st, launch); break;
+    }
+    if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
+    CombineArgs c;
+    c.part = launch.part;
+    c.meta = meta;
+    c.out_bf16 = static_cast<uint16_t *>(out_bf16);
+    c.out_q = out_q;
+    c.out_s = out_s;
+    c.M = M;
+    c.n_heads = n_heads;
+    c.n_chunks = a.n_chunks;
+    c.sigma = sigma;
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(M), dim3(kCombineThreads), 0, st, c);
+    return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" int bonsai_kv_commit(void *kv, int n_layers, int n_kv, int slots, int src_slot,
+                                int dst_slot, int n, void *stream) {
+    if (!kv || n_layers < 1 || n_kv < 1 || slots < 1 || n < 0 || src_slot < 0 || dst_slot < 0 ||
+        src_slot + n > slots || dst_slot + n > slots)
+        return BONSAI_DECODE_ERR_ARG;
+    if (n == 0) return BONSAI_DECODE_OK;
+    if (src_slot < dst_slot + n && dst_slot < src_slot + n) return BONSAI_DECODE_ERR_ARG;  // overlap
+    const int planes = 2 * n_layers * n_kv;
+    const long long work = (long long)planes * n * (kHd * 2 / 16);
+    if (work > 0x7fffffffLL) return BONSAI_DECODE_ERR_ARG;
+    hipLaunchKernelGGL(kv_commit_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<uint4 *>(kv), planes, slots,
+                       src_slot, dst_slot, n);
+    return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" int bonsai_draft_chain(const void *logits, int rows, int ld, int vocab, float threshold,
+                                  int32_t *tokens, float *conf, int32_t *accept, void *stream) {
+    if (!logits || !tokens || !conf || !accept) return BONSAI_DECODE_ERR_ARG;
+    if (rows < 1 || vocab < 1 || ld < vocab || ld % 8 != 0) return BONSAI_DECODE_ERR_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(draft_rows_kernel, dim3(rows), dim3(kDraftThreads), 0, st,
+                       static_cast<const uint16_t *>(logits), ld, vocab, tokens, conf);
+    if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
+    hipLaunchKernelGGL(draft_accept_kernel, dim3(1), dim3(64), 0, st, conf, rows, threshold, accept);
+    return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}

@@ -1,0 +1,97 @@
+"""End-to-end decode throughput of a random-init packed-ternary model on one MI355X.
+
+    python -m bitmtp_amd.decode_bench --model 1.7b            # 256-token prompt, 512 new
+    python -m bitmtp_amd.decode_bench --model 4b --prompt 512 --new 1024
+
+Reports tokens/s by the reference's timing contract (``timed_decode_tokens /
+decode_time``, prefill and the first token excluded; src/bonsai_sft/gpu/fast_generate.py:
+1001,1147-1148,1171) for greedy AR, for D8 hybrid decode with the default gate
+(threshold 0.9, chain 6) and for a forced-confidence run (threshold 0, chain 1) that
+exercises the wide draft graphs.  With random weights the logits are near-uniform, so the
+default gate verifies every iteration (draft width 9 + verify width 9, about one token per
+iteration); the forced run commits whole blocks.  Prompt ids are uniform random.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import time
+
+import numpy as np
+import torch
+
+from .generate import ar_generate, hybrid_generate
+from .model import BonsaiDecoder, qwen3_1p7b_args, qwen3_4b_args
+from .runtime import GraphAtlas
+
+MODELS = {"1.7b": qwen3_1p7b_args, "4b": qwen3_4b_args}
+
+
+def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens: int = 512,
+                     seed: int = 2, repeats: int = 2, device: str = "cuda:0",
+                     n_layers: int = 0) -> dict:
+    over = {"n_layers": n_layers} if n_layers else {}
+    args = MODELS[model_name](**over)
+    t0 = time.time()
+    model = BonsaiDecoder.random_init(args, seed=seed, device=device)
+    atlas = GraphAtlas(model, threshold=0.9)
+    torch.cuda.synchronize()
+    init_s = time.time() - t0
+    rng = np.random.default_rng(seed)
+    prompt = rng.integers(0, args.vocab_size, prompt_len).tolist()
+
+    def best(fn):
+        res = None
+        for _ in range(repeats + 1):   # the first pass also captures the graphs it needs
+            out, st = fn()
+            if res is None or st["decode_time"] < res[1]["decode_time"]:
+                res = (out, st)
+        return res
+
+    out_ar, st_ar = best(lambda: ar_generate(atlas, prompt, max_gen_len=new_tokens))
+    out_hy, st_hy = best(lambda: hybrid_generate(atlas, prompt, threshold=0.9,
+                                                 max_gen_len=new_tokens))
+    out_fc, st_fc = best(lambda: hybrid_generate(atlas, prompt, threshold=0.0, hybrid_m=1,
+                                                 max_gen_len=new_tokens))
+
+    def line(st, extra=()):
+        d = {"tokens_per_s": round(st["timed_decode_tokens"] / st["decode_time"], 1),
+             "decode_tokens": st["decode_tokens"], "decode_time_s": round(st["decode_time"], 4),
+             "prefill_time_s": round(st["prefill_time"], 4), "n_iters": st["n_iters"]}
+        for k in extra:
+            d[k] = st[k] if not isinstance(st[k], float) else round(st[k], 3)
+        return d
+
+    hy_keys = ("committed_per_iter", "n_conf_path", "n_verify_path", "accept_rate")
+    res = {
+        "model": f"random-init Qwen3-{model_name}-shaped T2-g128, {args.n_layers} layers, "
+                 f"dim {args.dim}, vocab {args.vocab_size}, packed T2 head",
+        "prompt_tokens": prompt_len, "new_tokens": new_tokens, "block_size": args.block_size,
+        "weight_bytes_per_step": model.weight_bytes_per_step(),
+        "init_s": round(init_s, 1),
+        "ar": line(st_ar),
+        "hybrid_d8_thr0.9_m6": line(st_hy, hy_keys),
+        "hybrid_d8_forced_confidence": line(st_fc, hy_keys),
+        "graphs_captured": sorted(f"{m}/{s}/{r}" for (m, s, r) in atlas.graphs),
+    }
+    ar_step_us = 1e6 * st_ar["decode_time"] / max(1, st_ar["timed_decode_tokens"])
+    res["ar"]["us_per_step"] = round(ar_step_us, 1)
+    res["ar"]["weight_stream_gbps"] = round(res["weight_bytes_per_step"] / ar_step_us / 1e3, 1)
+    return res
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--model", choices=sorted(MODELS), default="1.7b")
+    ap.add_argument("--prompt", type=int, default=256)
+    ap.add_argument("--new", type=int, default=512)
+    ap.add_argument("--seed", type=int, default=2)
+    ap.add_argument("--repeats", type=int, default=2)
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = model's)")
+    a = ap.parse_args()
+    print(json.dumps(run_decode_bench(a.model, a.prompt, a.new, a.seed, a.repeats,
+                                      n_layers=a.layers)))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,181 @@
+"""ctypes binding of ``decode_ops/libbonsai_decode.so``: the ops between the packed GEMVs
+of one captured decode step (include/bonsai_decode.h).  They take pre-allocated
+tensors and launch on the current stream, so all of them can be captured in a graph.
+
+No fallback: a missing library raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+HEAD_DIM = 128
+MAX_WIDTH = 32
+ATTN_CHUNK = 64
+
+_lib = None
+
+
+def decode_lib_path() -> str:
+    return os.path.join(_HERE, "decode_ops", "libbonsai_decode.so")
+
+
+def load_decode_kernel() -> None:
+    global _lib
+    so = decode_lib_path()
+    if not os.path.exists(so):
+        raise RuntimeError(
+            f"{so} is missing: build the gfx950 libraries with `python -m bitmtp_amd.build` "
+            "(there is no fallback implementation)")
+    lib = ctypes.CDLL(so)
+    vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    lib.bonsai_qk_norm_rope_kv_write.argtypes = [vp, vp, vp, cf, vp, vp, vp, vp, vp, vp,
+                                                 ci, ci, ci, ci, ci, ci, vp]
+    lib.bonsai_qk_norm_rope_kv_write.restype = ci
+    lib.bonsai_decode_attention_scratch_bytes.argtypes = [ci, ci, ci]
+    lib.bonsai_decode_attention_scratch_bytes.restype = ctypes.c_int64
+    lib.bonsai_decode_attention.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, cf,
+                                            ci, ci, ci, ci, ci, vp]
+    lib.bonsai_decode_attention.restype = ci
+    lib.bonsai_kv_commit.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
+    lib.bonsai_kv_commit.restype = ci
+    lib.bonsai_draft_chain.argtypes = [vp, ci, ci, ci, cf, vp, vp, vp, vp]
+    lib.bonsai_draft_chain.restype = ci
+    _lib = lib
+
+
+def decode_lib() -> ctypes.CDLL:
+    if _lib is None:
+        load_decode_kernel()
+    return _lib
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(device: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _need(cond: bool, what: str) -> None:
+    if not cond:
+        raise RuntimeError(what)
+
+
+def _check(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+    _need(t.is_cuda and t.is_contiguous() and t.dtype == dtype,
+          f"{name} must be a contiguous {dtype} CUDA tensor")
+
+
+def qk_norm_rope_kv_write(xqkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: torch.Tensor,
+                          eps: float, cos: torch.Tensor, sin: torch.Tensor,
+                          positions: torch.Tensor, q_out: torch.Tensor, k_layer: torch.Tensor,
+                          v_layer: torch.Tensor, n_heads: int, n_kv: int, write_slot: int) -> None:
+    """Per-head q/k RMSNorm + RoPE + KV write (reference: model.py:388-436).
+
+    ``xqkv`` bf16 ``[M, (n_heads+2 n_kv)*128]``; ``k_layer``/``v_layer`` bf16
+    ``[n_kv, slots, 128]``; ``q_out`` bf16 ``[M, n_heads, 128]``; ``positions`` int32 ``[M]``.
+    """
+    m = xqkv.shape[0]
+    for t, name in ((xqkv, "xqkv"), (q_norm_w, "q_norm_w"), (k_norm_w, "k_norm_w"), (cos, "cos"),
+                    (sin, "sin"), (q_out, "q_out"), (k_layer, "k_layer"), (v_layer, "v_layer")):
+        _check(t, torch.bfloat16, name)
+    _check(positions, torch.int32, "positions")
+    _need(xqkv.shape == (m, (n_heads + 2 * n_kv) * HEAD_DIM), "xqkv shape mismatch")
+    _need(q_out.shape == (m, n_heads, HEAD_DIM), "q_out shape mismatch")
+    _need(k_layer.shape == v_layer.shape and k_layer.dim() == 3 and k_layer.shape[0] == n_kv
+          and k_layer.shape[2] == HEAD_DIM, "KV layer shape mismatch")
+    _need(cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == HEAD_DIM,
+          "RoPE table shape mismatch")
+    _need(positions.numel() == m and q_norm_w.numel() == HEAD_DIM and k_norm_w.numel() == HEAD_DIM,
+          "positions / norm weight size mismatch")
+    slots = k_layer.shape[1]
+    with torch.cuda.device(xqkv.device):
+        rc = decode_lib().bonsai_qk_norm_rope_kv_write(
+            _ptr(xqkv), _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(cos), _ptr(sin),
+            _ptr(positions), _ptr(q_out), _ptr(k_layer), _ptr(v_layer), m, n_heads, n_kv, slots,
+            int(write_slot), cos.shape[0], _stream(xqkv.device))
+    _need(rc == 0, f"bonsai_qk_norm_rope_kv_write failed with status {rc}")
+
+
+def attention_scratch_bytes(m: int, n_heads: int, slots: int) -> int:
+    return int(decode_lib().bonsai_decode_attention_scratch_bytes(m, n_heads, slots))
+
+
+def decode_attention(q: torch.Tensor, k_layer: torch.Tensor, v_layer: torch.Tensor,
+                     meta: torch.Tensor, scratch: torch.Tensor, sigma: int,
+                     out_bf16: Optional[torch.Tensor] = None,
+                     out_q: Optional[torch.Tensor] = None, out_s: Optional[torch.Tensor] = None,
+                     scale: Optional[float] = None) -> None:
+    """Attention of the M new rows over the shared KV under the step descriptor ``meta``
+    (int32 ``[2+M]``: cache_len, hidden slot or -1, one workspace-visibility word per row),
+    optionally followed by the per-token quantisation of the result
+    (reference: model.py:996-1005, fast_runtime.py:391-465)."""
+    _check(q, torch.bfloat16, "q")
+    _check(k_layer, torch.bfloat16, "k_layer")
+    _check(v_layer, torch.bfloat16, "v_layer")
+    _check(meta, torch.int32, "meta")
+    m, n_heads = q.shape[0], q.shape[1]
+    n_kv, slots = k_layer.shape[0], k_layer.shape[1]
+    _need(q.dim() == 3 and q.shape[2] == HEAD_DIM, "q must be [M, n_heads, 128]")
+    _need(k_layer.shape == v_layer.shape and k_layer.shape[2] == HEAD_DIM, "KV layer shape mismatch")
+    _need(meta.numel() >= 2 + m, "meta needs 2 + M entries")
+    _need(scratch.is_cuda and scratch.is_contiguous()
+          and scratch.numel() * scratch.element_size() >= attention_scratch_bytes(m, n_heads, slots),
+          "attention scratch too small")
+    if out_bf16 is not None:
+        _check(out_bf16, torch.bfloat16, "out_bf16")
+        _need(out_bf16.numel() == m * n_heads * HEAD_DIM, "out_bf16 size mismatch")
+    if out_q is not None or out_s is not None:
+        _need(out_q is not None and out_s is not None, "out_q and out_s come together")
+        _check(out_q, torch.int8, "out_q")
+        _check(out_s, torch.float32, "out_s")
+        _need(out_q.numel() == m * n_heads * HEAD_DIM and out_s.numel() == m, "out_q/out_s size mismatch")
+    if scale is None:
+        scale = 1.0 / math.sqrt(HEAD_DIM)
+    with torch.cuda.device(q.device):
+        rc = decode_lib().bonsai_decode_attention(
+            _ptr(q), _ptr(k_layer), _ptr(v_layer), _ptr(meta), _ptr(scratch), _ptr(out_bf16),
+            _ptr(out_q), _ptr(out_s), float(scale), m, n_heads, n_kv, slots, int(sigma),
+            _stream(q.device))
+    _need(rc == 0, f"bonsai_decode_attention failed with status {rc}")
+
+
+def kv_commit(kv: torch.Tensor, src_slot: int, dst_slot: int, n: int) -> None:
+    """Copy ``n`` rows of every layer / kv head from slot ``src_slot`` to ``dst_slot`` of a
+    shared buffer ``[2, n_layers, n_kv, slots, 128]`` (reference: fast_runtime.py:467-508)."""
+    _check(kv, torch.bfloat16, "kv")
+    _need(kv.dim() == 5 and kv.shape[0] == 2 and kv.shape[4] == HEAD_DIM,
+          "kv must be [2, n_layers, n_kv, slots, 128]")
+    if n <= 0:
+        return
+    with torch.cuda.device(kv.device):
+        rc = decode_lib().bonsai_kv_commit(_ptr(kv), kv.shape[1], kv.shape[2], kv.shape[3],
+                                           int(src_slot), int(dst_slot), int(n), _stream(kv.device))
+    _need(rc == 0, f"bonsai_kv_commit failed with status {rc}")
+
+
+def draft_chain(logits: torch.Tensor, vocab: int, threshold: float, tokens: torch.Tensor,
+                conf: torch.Tensor, accept: torch.Tensor) -> None:
+    """Row argmax, confidence ``exp(max - logsumexp)`` and the accepted-prefix length
+    ``1 + longest prefix of rows 1.. with conf > threshold`` (reference:
+    fast_generate.py:111-130).  ``logits`` bf16 ``[rows, ld]``; outputs are pre-allocated
+    int32 ``[rows]``, fp32 ``[rows]`` and int32 ``[2]``."""
+    _check(logits, torch.bfloat16, "logits")
+    _check(tokens, torch.int32, "tokens")
+    _check(conf, torch.float32, "conf")
+    _check(accept, torch.int32, "accept")
+    rows, ld = logits.shape
+    _need(tokens.numel() >= rows and conf.numel() >= rows and accept.numel() >= 2,
+          "draft_chain output buffers too small")
+    with torch.cuda.device(logits.device):
+        rc = decode_lib().bonsai_draft_chain(_ptr(logits), rows, ld, int(vocab), float(threshold),
+                                             _ptr(tokens), _ptr(conf), _ptr(accept),
+                                             _stream(logits.device))
+    _need(rc == 0, f"bonsai_draft_chain failed with status {rc}")

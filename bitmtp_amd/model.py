@@ -1,0 +1,392 @@
+"""Packed-ternary Bonsai (Qwen3-shaped) decoder for MI355X: weights and the one
+fixed-shape decode step that the graph atlas captures.
+
+The step is the reference's fully kernelised graph forward
+(``Transformer.forward_sdlm_decode_graph_kernel``, src/bonsai_sft/gpu/model.py:1386-1403,
+with ``TransformerBlock.forward_sdlm_graph_kernel`` :1112-1137,
+``Attention.forward_sdlm_graph_kernel`` :958-1009 and
+``FeedForward.forward_merged_kernel`` :1053-1064), laid out MI355X-first: every op is
+one native launch on pre-allocated buffers,
+
+    embed gather -> [norm+quant | add+norm+quant] -> qkv GEMV -> qk-norm+RoPE+KV write
+    -> attention (+quant) -> o GEMV -> add+norm+quant -> gate|up GEMV -> SiLU*up+quant
+    -> down GEMV ... -> add+norm+quant (logit rows only) -> packed head GEMV
+    -> argmax / confidence chain
+
+so a replayed graph is 10 launches per layer and reads each packed weight once.
+PyTorch supplies device memory, the embedding gather and graph capture only.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from . import decode_ops, ops
+from .packing import GROUP_SIZE, _pack_fields
+
+HEAD_DIM = decode_ops.HEAD_DIM
+
+
+@dataclass
+class ModelArgs:
+    """Same fields and defaults as the reference ``ModelArgs`` (model.py:690-713)."""
+    dim: int = 2048
+    n_layers: int = 28
+    n_heads: int = 16
+    n_kv_heads: int = 8
+    head_dim: int = 128
+    ffn_dim: int = 6144
+    vocab_size: int = 151669
+    norm_eps: float = 1.0e-6
+    rope_theta: float = 1.0e6
+    rope_original_max: int = 8192
+    rope_factor: float = 4.0
+    rope_mscale: float = 1.0
+    rope_mscale_all_dim: float = 0.0
+    rope_beta_fast: float = 32.0
+    rope_beta_slow: float = 1.0
+    tie_word_embeddings: bool = True
+    use_kernel: bool = True
+    kernel_kind: str = "t2g128"
+    block_size: int = 8
+    causal_attn: bool = True
+    mask_token_id: int = 151654
+
+    @property
+    def q_dim(self) -> int:
+        return self.n_heads * self.head_dim
+
+    @property
+    def kv_dim(self) -> int:
+        return self.n_kv_heads * self.head_dim
+
+
+def qwen3_1p7b_args(**over) -> ModelArgs:
+    """Qwen3-1.7B shape: 28 layers, hidden 2048, 16 q / 8 kv heads x 128, ffn 6144."""
+    return ModelArgs(**{**dict(vocab_size=151936), **over})
+
+
+def qwen3_4b_args(**over) -> ModelArgs:
+    """Qwen3-4B shape: 36 layers, hidden 2560, 32 q / 8 kv heads x 128, ffn 9728."""
+    return ModelArgs(**{**dict(dim=2560, n_layers=36, n_heads=32, n_kv_heads=8, ffn_dim=9728,
+                               vocab_size=151936), **over})
+
+
+# ---------------------------------------------------------------------------
+# RoPE tables (reference: `_yarn_inv_freq`, `_yarn_attention_factor`, model.py:342-379,
+# and the lookup tables of `prepare_merged_weights`, model.py:950-955)
+# ---------------------------------------------------------------------------
+def yarn_inv_freq(head_dim: int, base: float, factor: float, original_max: int,
+                  beta_fast: float = 32.0, beta_slow: float = 1.0, device=None) -> torch.Tensor:
+    dim = head_dim
+    idx = torch.arange(0, dim, 2, device=device).float()
+    pos_freqs = base ** (idx / dim)
+    extrap = 1.0 / pos_freqs
+    interp = 1.0 / (factor * pos_freqs)
+
+    def correction_dim(rotations: float) -> float:
+        return (dim * math.log(original_max / (rotations * 2 * math.pi))) / (2 * math.log(base))
+
+    low = max(math.floor(correction_dim(beta_fast)), 0)
+    high = min(math.ceil(correction_dim(beta_slow)), dim - 1)
+    if low == high:
+        high += 0.001
+    ramp = ((torch.arange(dim // 2, device=device, dtype=torch.float32) - low) / (high - low)).clamp(0.0, 1.0)
+    keep = 1.0 - ramp
+    return interp * (1.0 - keep) + extrap * keep
+
+
+def yarn_attention_factor(scale: float, mscale: float = 1.0, mscale_all_dim: float = 0.0) -> float:
+    if scale <= 1.0:
+        return 1.0
+
+    def g(s, m):
+        return 0.1 * m * math.log(s) + 1.0
+    if mscale and mscale_all_dim:
+        return g(scale, mscale) / g(scale, mscale_all_dim)
+    return g(scale, mscale)
+
+
+def rope_tables(args: ModelArgs, max_positions: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
+    inv_freq = yarn_inv_freq(args.head_dim, args.rope_theta, args.rope_factor,
+                             args.rope_original_max, args.rope_beta_fast, args.rope_beta_slow,
+                             device=device)
+    mscale = yarn_attention_factor(args.rope_factor, args.rope_mscale, args.rope_mscale_all_dim)
+    pos = torch.arange(max_positions, device=device, dtype=torch.float32)
+    freqs = torch.outer(pos, inv_freq.float())
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return ((emb.cos() * mscale).to(torch.bfloat16).contiguous(),
+            (emb.sin() * mscale).to(torch.bfloat16).contiguous())
+
+
+# ---------------------------------------------------------------------------
+# Weights
+# ---------------------------------------------------------------------------
+@dataclass
+class PackedLinear:
+    weight: torch.Tensor        # int8 [N, K/4]
+    weight_scale: torch.Tensor  # bf16 [N, K/128]
+
+    @property
+    def out_features(self) -> int:
+        return self.weight.shape[0]
+
+    @property
+    def in_features(self) -> int:
+        return self.weight.shape[1] * 4
+
+
+@dataclass
+class LayerWeights:
+    """One block with q|k|v and gate|up already merged along the output rows
+    (reference: ``prepare_merged_weights``, model.py:931-956 and :1042-1051)."""
+    wqkv: PackedLinear
+    wo: PackedLinear
+    w_gu: PackedLinear
+    w_down: PackedLinear
+    input_layernorm: torch.Tensor           # bf16 [dim]
+    post_attention_layernorm: torch.Tensor  # bf16 [dim]
+    q_norm: torch.Tensor                    # bf16 [128]
+    k_norm: torch.Tensor                    # bf16 [128]
+
+
+def _random_packed(n: int, k: int, gen: torch.Generator, device) -> PackedLinear:
+    """i.i.d. ternary codes (p = 1/3 each) and log-normal(-4, 0.5) group scales."""
+    codes = torch.randint(1, 4, (n, k), generator=gen, device=device, dtype=torch.uint8)
+    packed = _pack_fields(codes, 2)
+    scale = torch.exp(torch.randn((n, k // GROUP_SIZE), generator=gen, device=device) * 0.5 - 4.0)
+    return PackedLinear(packed, scale.to(torch.bfloat16).contiguous())
+
+
+def head_rows_for(vocab: int) -> int:
+    """The packed head is padded to whole 128-row tiles (the reference pads 151669 to
+    151936, model.py:1227); pad rows carry zero scales and are never selected."""
+    return -(-vocab // 128) * 128
+
+
+class BonsaiDecoder:
+    """Weights of a packed-ternary decoder plus its step enqueue function."""
+
+    def __init__(self, args: ModelArgs, layers: List[LayerWeights], embed: torch.Tensor,
+                 norm: torch.Tensor, head: PackedLinear):
+        if args.head_dim != HEAD_DIM:
+            raise ValueError("only head_dim 128 is supported")
+        if args.kernel_kind != "t2g128":
+            raise ValueError("the decode harness covers the ternary t2g128 backbone")
+        if args.dim % GROUP_SIZE or args.ffn_dim % GROUP_SIZE or args.q_dim % GROUP_SIZE:
+            raise ValueError("dim, ffn_dim and n_heads*head_dim must be multiples of 128")
+        self.args = args
+        self.layers = layers
+        self.embed = embed          # bf16 [vocab, dim]
+        self.norm = norm            # bf16 [dim]
+        self.head = head            # packed [head_rows, dim/4]
+        self.device = embed.device
+        self.head_rows = head.out_features
+
+    # -- construction --------------------------------------------------------
+    @classmethod
+    def random_init(cls, args: ModelArgs, seed: int = 0, device="cuda") -> "BonsaiDecoder":
+        """Random ternary weights; the embedding is the dequantised tied head, as in a
+        converted checkpoint whose tied projection sits on the ternary grid
+        (reference: ``prepare_t2_lm_head``, model.py:1222-1243)."""
+        device = torch.device(device)
+        gen = torch.Generator(device=device)
+        gen.manual_seed(seed)
+        layers = []
+        for _ in range(args.n_layers):
+            def ln(n):
+                return (1.0 + 0.1 * torch.randn(n, generator=gen, device=device)).to(torch.bfloat16)
+            layers.append(LayerWeights(
+                wqkv=_random_packed(args.q_dim + 2 * args.kv_dim, args.dim, gen, device),
+                wo=_random_packed(args.dim, args.q_dim, gen, device),
+                w_gu=_random_packed(2 * args.ffn_dim, args.dim, gen, device),
+                w_down=_random_packed(args.dim, args.ffn_dim, gen, device),
+                input_layernorm=ln(args.dim), post_attention_layernorm=ln(args.dim),
+                q_norm=ln(HEAD_DIM), k_norm=ln(HEAD_DIM)))
+        rows = head_rows_for(args.vocab_size)
+        head = _random_packed(rows, args.dim, gen, device)
+        if rows > args.vocab_size:
+            head.weight_scale[args.vocab_size:] = 0
+        embed = dequantize_t2(head)[: args.vocab_size].contiguous()
+        norm = (1.0 + 0.1 * torch.randn(args.dim, generator=gen, device=device)).to(torch.bfloat16)
+        return cls(args, layers, embed, norm, head)
+
+    def weight_bytes_per_step(self) -> int:
+        """Packed weight + scale bytes one replay streams (head included)."""
+        total = 0
+        for lw in self.layers:
+            for p in (lw.wqkv, lw.wo, lw.w_gu, lw.w_down):
+                total += p.weight.numel() + 2 * p.weight_scale.numel()
+        return total + self.head.weight.numel() + 2 * self.head.weight_scale.numel()
+
+
+def dequantize_t2(p: PackedLinear) -> torch.Tensor:
+    """bf16 [N, K] = (code - 2) * group scale (reference: ``_unpack_to_bf16``, model.py:641-647)."""
+    b = p.weight.view(torch.uint8)
+    shifts = torch.arange(0, 8, 2, device=b.device, dtype=torch.uint8)
+    q = ((b.unsqueeze(-1) >> shifts) & 3).to(torch.int8) - 2
+    n = b.shape[0]
+    q = q.view(n, -1, GROUP_SIZE).to(torch.bfloat16)
+    return (q * p.weight_scale.unsqueeze(-1)).view(n, -1)
+
+
+# ---------------------------------------------------------------------------
+# The step
+# ---------------------------------------------------------------------------
+class Workspace:
+    """Intermediate buffers of one step, sized for the widest graph and shared by all
+    graphs (they replay one after another on one stream)."""
+
+    def __init__(self, args: ModelArgs, m_max: int, max_slots: int, head_rows: int, device):
+        bf, i8, f32 = torch.bfloat16, torch.int8, torch.float32
+
+        def buf(shape, dtype):
+            return torch.zeros(shape, dtype=dtype, device=device)
+        self.m_max = m_max
+        self.h = [buf((m_max, args.dim), bf), buf((m_max, args.dim), bf)]
+        self.a_q = buf((m_max, args.dim), i8)
+        self.a_s = buf((m_max,), f32)
+        self.xqkv = buf((m_max, args.q_dim + 2 * args.kv_dim), bf)
+        self.q = buf((m_max, args.n_heads, HEAD_DIM), bf)
+        nbytes = decode_ops.attention_scratch_bytes(m_max, args.n_heads, max_slots)
+        self.attn_scratch = buf((nbytes // 4,), f32)
+        self.o_q = buf((m_max, args.q_dim), i8)
+        self.o_s = buf((m_max,), f32)
+        self.attn_out = buf((m_max, args.dim), bf)
+        self.f_q = buf((m_max, args.dim), i8)
+        self.f_s = buf((m_max,), f32)
+        self.gu = buf((m_max, 2 * args.ffn_dim), bf)
+        self.i_q = buf((m_max, args.ffn_dim), i8)
+        self.i_s = buf((m_max,), f32)
+        self.ffn_out = buf((m_max, args.dim), bf)
+        self.h_last = buf((m_max, args.dim), bf)
+        self.l_q = buf((m_max, args.dim), i8)
+        self.l_s = buf((m_max,), f32)
+        self.logits = buf((m_max, head_rows), bf)
+
+
+@dataclass
+class StepIO:
+    """Per-graph inputs and outputs.  ``step_in`` is one int32 vector
+    ``[meta (2+M) | positions (M) | tokens (M)]`` so a replay needs a single
+    host-to-device copy; ``out`` is ``[argmax tokens (M) | accept (2) | conf bits (M)]``
+    so the results come back in a single device-to-host copy."""
+    M: int
+    step_in: torch.Tensor        # int32 [3M+2] device
+    step_in_host: torch.Tensor   # pinned mirror
+    out: torch.Tensor            # int32 [2M+2] device
+    out_host: torch.Tensor       # pinned mirror
+    uploaded: "torch.cuda.Event"  # recorded after each upload of step_in_host
+
+    @property
+    def meta(self) -> torch.Tensor:
+        return self.step_in[: 2 + self.M]
+
+    @property
+    def positions(self) -> torch.Tensor:
+        return self.step_in[2 + self.M: 2 + 2 * self.M]
+
+    @property
+    def tokens(self) -> torch.Tensor:
+        return self.step_in[2 + 2 * self.M:]
+
+    @property
+    def tokens_out(self) -> torch.Tensor:
+        return self.out[: self.M]
+
+    @property
+    def accept(self) -> torch.Tensor:
+        return self.out[self.M: self.M + 2]
+
+    @property
+    def conf(self) -> torch.Tensor:
+        return self.out[self.M + 2:].view(torch.float32)
+
+    @classmethod
+    def allocate(cls, M: int, device) -> "StepIO":
+        return cls(M=M,
+                   step_in=torch.zeros(3 * M + 2, dtype=torch.int32, device=device),
+                   step_in_host=torch.zeros(3 * M + 2, dtype=torch.int32).pin_memory(),
+                   out=torch.zeros(2 * M + 2, dtype=torch.int32, device=device),
+                   out_host=torch.zeros(2 * M + 2, dtype=torch.int32).pin_memory(),
+                   uploaded=torch.cuda.Event())
+
+
+def _vp(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _gemv(a_q: torch.Tensor, a_s: torch.Tensor, w: PackedLinear, out: torch.Tensor, m: int,
+          stream: ctypes.c_void_p) -> None:
+    rc = ops.t2_lib().t2g128_gemv_ex(_vp(a_q), _vp(w.weight), _vp(out), _vp(a_s),
+                                     _vp(w.weight_scale), m, w.out_features, w.in_features,
+                                     ops.OUT_BF16, ops.SCALE_BF16, stream)
+    if rc != 0:
+        raise RuntimeError(f"t2g128_gemv_ex failed with status {rc}")
+
+
+def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tensor, sigma: int,
+                 rope: Tuple[torch.Tensor, torch.Tensor], logits_start: int, logits_end: int,
+                 threshold: float) -> None:
+    """Enqueue one width-``io.M`` step on the current stream.
+
+    ``kv`` is the shared buffer ``[2, n_layers, n_kv, slots, 128]``; the new rows go to
+    slots ``sigma .. sigma+M-1``.  Logit rows ``[logits_start, logits_end)`` are projected
+    through the packed head; their argmax, confidence and accepted-prefix length land in
+    ``io.tokens_out / io.conf / io.accept`` (rows counted from ``logits_start``).
+    """
+    args = model.args
+    M = io.M
+    dim = args.dim
+    eps = float(args.norm_eps)
+    actq = ops.actq_lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(model.device).cuda_stream)
+    cos, sin = rope
+
+    def check(rc: int, what: str) -> None:
+        if rc != 0:
+            raise RuntimeError(f"{what} failed with status {rc}")
+
+    h_cur, h_nxt = ws.h[0][:M], ws.h[1][:M]
+    torch.index_select(model.embed, 0, io.tokens, out=h_cur)
+    for i, lw in enumerate(model.layers):
+        if i == 0:
+            check(actq.bonsai_rmsnorm_quant_int8(_vp(h_cur), _vp(lw.input_layernorm), eps,
+                                                 _vp(ws.a_q), _vp(ws.a_s), M, dim, stream),
+                  "bonsai_rmsnorm_quant_int8")
+        else:
+            check(actq.bonsai_add_rmsnorm_quant_int8(_vp(ws.ffn_out), _vp(h_cur),
+                                                     _vp(lw.input_layernorm), eps, _vp(h_nxt),
+                                                     _vp(ws.a_q), _vp(ws.a_s), M, dim, stream),
+                  "bonsai_add_rmsnorm_quant_int8")
+            h_cur, h_nxt = h_nxt, h_cur
+        _gemv(ws.a_q, ws.a_s, lw.wqkv, ws.xqkv, M, stream)
+        decode_ops.qk_norm_rope_kv_write(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
+                                         io.positions, ws.q[:M], kv[0, i], kv[1, i],
+                                         args.n_heads, args.n_kv_heads, sigma)
+        decode_ops.decode_attention(ws.q[:M], kv[0, i], kv[1, i], io.meta, ws.attn_scratch, sigma,
+                                    out_q=ws.o_q[:M], out_s=ws.o_s[:M])
+        _gemv(ws.o_q, ws.o_s, lw.wo, ws.attn_out, M, stream)
+        check(actq.bonsai_add_rmsnorm_quant_int8(_vp(h_cur), _vp(ws.attn_out),
+                                                 _vp(lw.post_attention_layernorm), eps, _vp(h_nxt),
+                                                 _vp(ws.f_q), _vp(ws.f_s), M, dim, stream),
+              "bonsai_add_rmsnorm_quant_int8")
+        h_cur, h_nxt = h_nxt, h_cur
+        _gemv(ws.f_q, ws.f_s, lw.w_gu, ws.gu, M, stream)
+        check(actq.bonsai_silu_mul_quant_int8(_vp(ws.gu), _vp(ws.i_q), _vp(ws.i_s), M,
+                                              args.ffn_dim, stream),
+              "bonsai_silu_mul_quant_int8")
+        _gemv(ws.i_q, ws.i_s, lw.w_down, ws.ffn_out, M, stream)
+
+    rows = logits_end - logits_start
+    check(actq.bonsai_add_rmsnorm_quant_int8(_vp(ws.ffn_out[logits_start:]), _vp(h_cur[logits_start:]),
+                                             _vp(model.norm), eps, _vp(ws.h_last), _vp(ws.l_q),
+                                             _vp(ws.l_s), rows, dim, stream),
+          "bonsai_add_rmsnorm_quant_int8")
+    _gemv(ws.l_q, ws.l_s, model.head, ws.logits, rows, stream)
+    decode_ops.draft_chain(ws.logits[:rows], args.vocab_size, threshold, io.tokens_out, io.conf,
+                           io.accept)

@@ -1,0 +1,105 @@
+/* C ABI of libbonsai_decode.so: the per-layer ops that sit between the packed GEMVs
+ * of one captured decode step on gfx950 (MI355X).
+ *
+ * The reference runs these steps as torch.compile'd Python inside its CUDA graphs:
+ *   - split + per-head q/k RMSNorm + RoPE + in-place KV write at a fixed offset
+ *     (`_fused_qkv_qknorm_rope_kv_write`, src/bonsai_sft/gpu/model.py:388-436);
+ *   - attention of the M new rows over the shared KV buffer
+ *     (`Attention.forward_sdlm_graph_kernel`, src/bonsai_sft/gpu/model.py:996-1003)
+ *     under the additive mask that `GraphAtlas.prepare_step` rebuilds every step
+ *     (src/bonsai_sft/gpu/fast_runtime.py:391-421,443-465), followed by the per-token
+ *     quantisation of the o_proj input (src/bonsai_sft/gpu/model.py:1004-1005);
+ *   - the argmax/confidence chain over the draft logits (`_fused_draft_chain`,
+ *     src/bonsai_sft/gpu/fast_generate.py:111-130) and the verifier's row argmax
+ *     (src/bonsai_sft/gpu/fast_generate.py:1073).
+ *
+ * Every entry point only enqueues kernels on `stream`: no allocation, no
+ * synchronisation, no memset, so all of them may be captured into a HIP graph.
+ * They return BONSAI_DECODE_OK or an error code and never print.
+ *
+ * KV layout (one layer): K and V are separate bf16 arrays [n_kv][slots][128];
+ * slot t < sigma holds history position t, slots sigma .. sigma+M-1 are the
+ * workspace the current step writes (src/bonsai_sft/gpu/fast_runtime.py:130-138).
+ *
+ * Step descriptor `meta` (int32, device memory, written by the host before each
+ * replay; it replaces the reference's dense [1,1,M,sigma+M] additive mask):
+ *   meta[0]      cache_len   history slots [0, cache_len) are visible to every row
+ *   meta[1]      hide        one history slot hidden from every row, or -1
+ *   meta[2 + r]  bit j set   row r sees workspace slot sigma + j      (r, j < M <= 32)
+ * A row that sees nothing at all yields zeros (the reference lets such padding rows
+ * look at slot 0 instead; their output is discarded either way).
+ */
+#ifndef BONSAI_DECODE_H
+#define BONSAI_DECODE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BONSAI_DECODE_OK 0
+#define BONSAI_DECODE_ERR_ARG 1
+#define BONSAI_DECODE_ERR_LAUNCH 2
+
+#define BONSAI_HEAD_DIM 128     /* the only head size of the Bonsai/Qwen3 family */
+#define BONSAI_MAX_WIDTH 32     /* rows per step (the reference uses at most 17) */
+#define BONSAI_ATTN_CHUNK 64    /* KV slots per attention work item */
+
+/* Replaces `_fused_qkv_qknorm_rope_kv_write` (src/bonsai_sft/gpu/model.py:388-436).
+ *   xqkv      bf16 [M, (n_heads + 2 n_kv) * 128]   merged q|k|v GEMV output
+ *   q_norm_w, k_norm_w  bf16 [128]
+ *   cos, sin  bf16 [max_pos, 128]                  RoPE tables (model.py:950-955)
+ *   positions int32 [M] (device)                   clamped into [0, max_pos)
+ *   q_out     bf16 [M, n_heads, 128]
+ *   k_layer, v_layer  bf16 [n_kv, slots, 128]      rows written at slot write_slot + m
+ * Rounding points are the eager ones of the reference expression:
+ *   n = bf16(w * bf16(fp32(x) * rs)),  rs = 1/sqrt(mean(fp32(x)^2) + eps)
+ *   out = bf16( bf16(n * cos) + bf16(rotate_half(n) * sin) );  V is copied. */
+int bonsai_qk_norm_rope_kv_write(const void *xqkv, const void *q_norm_w, const void *k_norm_w,
+                                 float eps, const void *cos_table, const void *sin_table,
+                                 const int32_t *positions, void *q_out, void *k_layer,
+                                 void *v_layer, int M, int n_heads, int n_kv, int slots,
+                                 int write_slot, int max_pos, void *stream);
+
+/* Bytes of scratch `bonsai_decode_attention` needs for the given shape. */
+int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int slots);
+
+/* Replaces the attention of `forward_sdlm_graph_kernel` (src/bonsai_sft/gpu/model.py:996-1003)
+ * and the quantisation of its output (model.py:1004).
+ *   q        bf16 [M, n_heads, 128]
+ *   k_layer, v_layer  bf16 [n_kv, slots, 128]
+ *   meta     int32 [2 + M] (device), see above; sigma = first workspace slot
+ *   scratch  at least bonsai_decode_attention_scratch_bytes(M, n_heads, slots) bytes
+ *   out_bf16 bf16 [M, n_heads*128] or NULL
+ *   out_q    int8 [M, n_heads*128] and out_s fp32 [M] (multiplier 127/absmax), or both NULL
+ * softmax(q k^T * scale + mask) v per head with fp32 accumulation; the KV read is
+ * bounded by cache_len + M, not by the buffer size.  Compared with a fp32 reference
+ * within rtol 2e-2 / atol 2e-3 on the bf16 output (bf16 inputs, fp32 softmax). */
+int bonsai_decode_attention(const void *q, const void *k_layer, const void *v_layer,
+                            const int32_t *meta, void *scratch, void *out_bf16, int8_t *out_q,
+                            float *out_s, float scale, int M, int n_heads, int n_kv, int slots,
+                            int sigma, void *stream);
+
+/* Copies n KV rows of every layer and kv head from slot src to slot dst inside one
+ * shared buffer [2, n_layers, n_kv, slots, 128] bf16 (commit_kv / commit_kv_from_verify,
+ * src/bonsai_sft/gpu/fast_runtime.py:467-508).  Source and destination ranges must
+ * not overlap. */
+int bonsai_kv_commit(void *kv, int n_layers, int n_kv, int slots, int src_slot, int dst_slot,
+                     int n, void *stream);
+
+/* Row argmax + confidence of the draft logits (`_fused_draft_chain`,
+ * src/bonsai_sft/gpu/fast_generate.py:111-130):
+ *   logits bf16 [rows, ld], the first `vocab` columns of each row are used
+ *   tokens int32 [rows]   argmax (lowest index among equal maxima)
+ *   conf   fp32 [rows]    exp(max - logsumexp(row)) in fp32
+ *   accept int32 [2]      accept[0] = 1 + longest prefix of rows 1.. with conf > threshold
+ *                         (NaN compares false); accept[1] = rows
+ * One launch for all rows. */
+int bonsai_draft_chain(const void *logits, int rows, int ld, int vocab, float threshold,
+                       int32_t *tokens, float *conf, int32_t *accept, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BONSAI_DECODE_H */

@@ -1,5 +1,5 @@
-"""The C-ABI libraries load without a GPU and export every entry point that
-include/bonsai_gemv.h declares (no compute call is made here)."""
+"""The C-ABI libraries load without a GPU and export every entry point that the headers
+under include/ declare (no compute call is made here)."""
 import ctypes
 import os
 import re
@@ -7,20 +7,25 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "bonsai_gemv.h")
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("bonsai_gemv.h", "bonsai_decode.h")]
 
 
 def declared_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(?:int|void)\s+([a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in HEADERS:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(?:int|void|int64_t)\s+([a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 @pytest.fixture(scope="module")
 def libs():
     from bitmtp_amd import build, ops
     build.build_all(verbose=False)  # compiles only what is missing or out of date
-    paths = [ops.t2_lib_path(), ops.q1_lib_path(), ops.actq_lib_path()]
+    from bitmtp_amd import decode_ops
+    paths = [ops.t2_lib_path(), ops.q1_lib_path(), ops.actq_lib_path(),
+             decode_ops.decode_lib_path()]
     assert all(os.path.exists(p) for p in paths)
     return [ctypes.CDLL(p) for p in paths]
 
@@ -40,7 +45,7 @@ def test_every_declared_symbol_is_exported(libs):
 def test_reference_loader_view_of_the_libraries(libs):
     """What the reference's ctypes loaders touch (src/bonsai_sft/gpu/model.py:70-93,
     206-219): both Q1 symbols in libbonsai_q1.so, the T2 symbol in libbonsai_t2.so."""
-    t2, q1, _ = libs
+    t2, q1 = libs[0], libs[1]
     assert hasattr(t2, "t2g128_int8xint2_linear")
     assert hasattr(q1, "q1g128_int8xint1_linear") and hasattr(q1, "q1g128_w1a16_linear")
     from bitmtp_amd import ops
@@ -57,3 +62,17 @@ def test_python_binding_sets_argtypes():
     assert ops.t2_lib().t2g128_int8xint2_linear.restype is None
     assert len(ops.q1_lib().q1g128_w1a16_linear.argtypes) == 8
     assert len(ops.t2_lib().t2g128_gemv_ex.argtypes) == 11
+
+
+def test_decode_library_exports_and_binding(libs):
+    assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["bonsai_decode.h", "bonsai_gemv.h"]
+    dec = libs[3]
+    for name in ("bonsai_qk_norm_rope_kv_write", "bonsai_decode_attention",
+                 "bonsai_decode_attention_scratch_bytes", "bonsai_kv_commit", "bonsai_draft_chain"):
+        assert name in declared_functions() and hasattr(dec, name)
+    from bitmtp_amd import decode_ops
+    decode_ops.load_decode_kernel()
+    assert len(decode_ops.decode_lib().bonsai_decode_attention.argtypes) == 15
+    # host-only query: partials are [M][heads][chunks][132] fp32
+    assert decode_ops.attention_scratch_bytes(9, 16, 1024 + 17) == 9 * 16 * 17 * 132 * 4
+    assert decode_ops.attention_scratch_bytes(0, 16, 64) == 0

@@ -1,0 +1,343 @@
+"""GPU tests of the decode harness: the ops between the GEMVs against the decode oracle,
+one whole captured step against the CPU composition of the oracles, and the system
+invariants of the generation loops (fast_generate.py:611-657,1151-1162).
+
+Tolerances: q/k-norm + RoPE, KV commit and the quantisation after attention are bit-exact;
+attention (bf16 inputs, fp32 online softmax on the GPU, float64 in the oracle) is compared
+on its bf16 output with rtol 2e-2 / atol 2e-3; whole-step logits with atol 6e-2 * max|logit|.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import bf16_bits, bf16_ordinal
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _bf16_from_bits(bits: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def _rand_bf16(rng, shape, std=1.0):
+    return torch.from_numpy(rng.normal(0, std, shape).astype(np.float32)).to(torch.bfloat16)
+
+
+@pytest.fixture(scope="module")
+def DO():
+    from oracle import decode_oracle
+    from oracle import oracle as O
+    O.build()
+    return decode_oracle
+
+
+# ---------------------------------------------------------------- qk norm + rope
+@pytest.mark.parametrize("M,n_heads,n_kv", [(1, 16, 8), (9, 16, 8), (17, 32, 8), (5, 3, 1)])
+def test_qk_norm_rope_bit_exact(DO, M, n_heads, n_kv):
+    from bitmtp_amd import decode_ops
+    from bitmtp_amd.model import ModelArgs, rope_tables
+    rng = np.random.default_rng(M * 100 + n_heads)
+    slots, write = 64, 40
+    xqkv = _rand_bf16(rng, (M, (n_heads + 2 * n_kv) * 128), 2.0)
+    qw = (1 + 0.1 * _rand_bf16(rng, (128,)).float()).to(torch.bfloat16)
+    kw = (1 + 0.1 * _rand_bf16(rng, (128,)).float()).to(torch.bfloat16)
+    cos_t, sin_t = rope_tables(ModelArgs(), 512, "cpu")
+    positions = torch.from_numpy(rng.integers(0, 512, M).astype(np.int32))
+    k_layer = _rand_bf16(rng, (n_kv, slots, 128))
+    v_layer = _rand_bf16(rng, (n_kv, slots, 128))
+    q_out = torch.zeros(M, n_heads, 128, dtype=torch.bfloat16)
+
+    d = [t.to(DEV) for t in (xqkv, qw, kw, cos_t, sin_t, positions, q_out, k_layer, v_layer)]
+    decode_ops.qk_norm_rope_kv_write(d[0], d[1], d[2], 1e-6, d[3], d[4], d[5], d[6], d[7], d[8],
+                                     n_heads, n_kv, write)
+    torch.cuda.synchronize()
+    q, k, v = DO.qk_norm_rope(bf16_bits(xqkv), bf16_bits(qw), bf16_bits(kw), 1e-6, bf16_bits(cos_t),
+                              bf16_bits(sin_t), positions.numpy(), n_heads, n_kv)
+    assert np.array_equal(bf16_bits(d[6]), q)
+    want_k = bf16_bits(k_layer).copy()
+    want_v = bf16_bits(v_layer).copy()
+    want_k[:, write:write + M] = k.transpose(1, 0, 2)
+    want_v[:, write:write + M] = v.transpose(1, 0, 2)
+    assert np.array_equal(bf16_bits(d[7]), want_k)      # also: no other slot was touched
+    assert np.array_equal(bf16_bits(d[8]), want_v)
+
+
+# ---------------------------------------------------------------- attention
+ATTN_CASES = [
+    # M, n_heads, n_kv, sigma, cache_len, role, n_pend
+    (1, 16, 8, 256, 0, "ar", 0),
+    (1, 16, 8, 256, 1, "ar", 0),
+    (1, 16, 8, 256, 200, "ar", 0),
+    (1, 32, 8, 1024, 777, "ar", 0),
+    (9, 16, 8, 256, 63, "verify", 0),
+    (9, 16, 8, 256, 64, "verify", 0),
+    (9, 32, 8, 1024, 1000, "verify", 0),
+    (9, 16, 8, 256, 100, "draft", 1),
+    (10, 16, 8, 256, 129, "draft", 2),
+    (12, 16, 8, 256, 55, "draft", 3),
+    (16, 16, 8, 1024, 500, "draft", 8),
+    (17, 32, 8, 256, 239, "draft", 9),
+    (16, 16, 8, 256, 0, "ar", 0),
+    (16, 16, 8, 256, 240, "ar", 0),
+    (5, 3, 1, 64, 30, "verify", 0),
+    (8, 16, 8, 256, 77, "draft", 0),
+]
+
+
+@pytest.mark.parametrize("M,n_heads,n_kv,sigma,cache_len,role,n_pend", ATTN_CASES)
+def test_attention_against_oracle(DO, oracle, M, n_heads, n_kv, sigma, cache_len, role, n_pend):
+    from bitmtp_amd import decode_ops, runtime
+    rng = np.random.default_rng(hash((M, n_heads, sigma, cache_len)) % (2 ** 31))
+    slots = sigma + 17
+    q = _rand_bf16(rng, (M, n_heads, 128), 1.5)
+    k = _rand_bf16(rng, (n_kv, slots, 128), 1.5)
+    v = _rand_bf16(rng, (n_kv, slots, 128), 1.0)
+    desc = runtime.step_descriptor(role, M, 8, cache_len, n_pend)
+    meta = torch.tensor(desc, dtype=torch.int32, device=DEV)
+    scratch = torch.empty(decode_ops.attention_scratch_bytes(M, n_heads, slots) // 4,
+                          dtype=torch.float32, device=DEV)
+    out = torch.zeros(M, n_heads * 128, dtype=torch.bfloat16, device=DEV)
+    out_q = torch.zeros(M, n_heads * 128, dtype=torch.int8, device=DEV)
+    out_s = torch.zeros(M, dtype=torch.float32, device=DEV)
+    print(f"attention case M={M} heads={n_heads}/{n_kv} sigma={sigma} cache_len={cache_len} {role}",
+          flush=True)
+    decode_ops.decode_attention(q.to(DEV), k.to(DEV), v.to(DEV), meta, scratch, sigma,
+                                out_bf16=out, out_q=out_q, out_s=out_s)
+    torch.cuda.synchronize()
+    vis = runtime.dense_visibility(desc, M, sigma)
+    # the oracle reads workspace rows where the kernel does: slots sigma..sigma+M-1
+    want = DO.attention(bf16_bits(q), bf16_bits(k), bf16_bits(v), vis, 1 / np.sqrt(128))
+    got = out.float().cpu().numpy().astype(np.float64)
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-3)
+    # quantisation of the kernel's own bf16 result is exact
+    wq, wsc = oracle.c_act_quant(out.float().cpu().numpy())
+    assert np.array_equal(out_q.cpu().numpy(), wq)
+    assert np.array_equal(out_s.cpu().numpy(), wsc)
+
+
+def test_attention_row_without_visible_slot_is_zero(DO):
+    from bitmtp_amd import decode_ops
+    M, n_heads, n_kv, sigma = 4, 2, 1, 64
+    rng = np.random.default_rng(0)
+    q = _rand_bf16(rng, (M, n_heads, 128)).to(DEV)
+    k = _rand_bf16(rng, (n_kv, sigma + M, 128)).to(DEV)
+    v = _rand_bf16(rng, (n_kv, sigma + M, 128)).to(DEV)
+    meta = torch.tensor([0, -1, 1, 0, 0b101, 0], dtype=torch.int32, device=DEV)
+    scratch = torch.empty(decode_ops.attention_scratch_bytes(M, n_heads, sigma + M) // 4,
+                          dtype=torch.float32, device=DEV)
+    out = torch.full((M, n_heads * 128), 7.0, dtype=torch.bfloat16, device=DEV)
+    decode_ops.decode_attention(q, k, v, meta, scratch, sigma, out_bf16=out)
+    torch.cuda.synchronize()
+    o = out.float().cpu()
+    assert torch.all(o[1] == 0) and torch.all(o[3] == 0)
+    # row 0 sees only workspace row 0: its output is that V row
+    assert torch.equal(out[0].view(n_heads, 128)[0].cpu(), v[0, sigma].cpu())
+    assert torch.any(o[2] != 0)
+
+
+def test_kv_commit_moves_exactly_the_rows():
+    from bitmtp_amd import decode_ops
+    rng = np.random.default_rng(1)
+    kv = _rand_bf16(rng, (2, 3, 2, 40, 128)).to(DEV)
+    want = kv.clone()
+    want[:, :, :, 5:9] = want[:, :, :, 31:35]
+    decode_ops.kv_commit(kv, 31, 5, 4)
+    torch.cuda.synchronize()
+    assert torch.equal(kv, want)
+    with pytest.raises(RuntimeError):
+        decode_ops.kv_commit(kv, 5, 7, 4)      # overlapping ranges
+    decode_ops.kv_commit(kv, 5, 7, 0)          # nothing to do
+
+
+@pytest.mark.parametrize("rows,vocab,ld", [(1, 151936, 151936), (8, 151669, 151936), (9, 1000, 1024),
+                                           (3, 37, 40)])
+def test_draft_chain_kernel(DO, rows, vocab, ld):
+    from bitmtp_amd import decode_ops
+    rng = np.random.default_rng(rows + vocab)
+    logits = _rand_bf16(rng, (rows, ld), 2.0)
+    # make some rows confident, plant a tie and poison the padding columns
+    for r in range(1, rows, 2):
+        logits[r, (r * 7919) % vocab] = 30.0
+    if rows > 2 and vocab > 20:
+        logits[2, 5] = 25.0
+        logits[2, 17] = 25.0
+    logits[:, vocab:] = 100.0
+    tokens = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    conf = torch.zeros(rows, dtype=torch.float32, device=DEV)
+    accept = torch.zeros(2, dtype=torch.int32, device=DEV)
+    decode_ops.draft_chain(logits.to(DEV), vocab, 0.9, tokens, conf, accept)
+    torch.cuda.synchronize()
+    wt, wc, wn = DO.draft_chain(logits[:, :vocab].float().numpy(), 0.9)
+    assert tokens.cpu().tolist() == wt.tolist()
+    np.testing.assert_allclose(conf.cpu().numpy(), wc, rtol=2e-3, atol=1e-6)
+    assert accept.cpu().tolist() == [wn, rows]
+
+
+# ---------------------------------------------------------------- whole step and loops
+def _tiny_args(**over):
+    from bitmtp_amd.model import ModelArgs
+    base = dict(dim=512, n_layers=2, n_heads=4, n_kv_heads=2, ffn_dim=1024, vocab_size=1000,
+                mask_token_id=999)
+    base.update(over)
+    return ModelArgs(**base)
+
+
+@pytest.fixture(scope="module")
+def tiny():
+    from bitmtp_amd.model import BonsaiDecoder
+    from bitmtp_amd.runtime import GraphAtlas
+    model = BonsaiDecoder.random_init(_tiny_args(), seed=11, device=DEV)
+    atlas = GraphAtlas(model, segment_ladder=(64, 256), threshold=0.9)
+    return model, atlas
+
+
+def _oracle_weights(model, atlas):
+    def pl(p):
+        return (p.weight.cpu().numpy().view(np.uint8), bf16_bits(p.weight_scale))
+    a = model.args
+    return {
+        "embed": bf16_bits(model.embed), "norm": bf16_bits(model.norm), "head": pl(model.head),
+        "cos": bf16_bits(atlas.rope[0]), "sin": bf16_bits(atlas.rope[1]), "eps": a.norm_eps,
+        "n_heads": a.n_heads, "n_kv": a.n_kv_heads,
+        "layers": [{
+            "wqkv": pl(l.wqkv), "wo": pl(l.wo), "w_gu": pl(l.w_gu), "w_down": pl(l.w_down),
+            "input_layernorm": bf16_bits(l.input_layernorm),
+            "post_attention_layernorm": bf16_bits(l.post_attention_layernorm),
+            "q_norm": bf16_bits(l.q_norm), "k_norm": bf16_bits(l.k_norm)} for l in model.layers],
+    }
+
+
+@pytest.mark.parametrize("role,M,n_pend", [("ar", 1, 0), ("verify", 9, 0), ("draft", 12, 3),
+                                           ("ar", 16, 0)])
+def test_captured_step_against_cpu_composition(DO, tiny, role, M, n_pend):
+    from bitmtp_amd import runtime
+    model, atlas = tiny
+    sigma, cache_len = 64, 21
+    rng = np.random.default_rng(M)
+    kv = atlas.kv(sigma)
+    kv.copy_(_rand_bf16(rng, tuple(kv.shape), 0.5).to(DEV))
+    kv_bits = bf16_bits(kv)
+    tokens = rng.integers(0, model.args.vocab_size, M).tolist()
+    positions = [cache_len + i for i in range(M)]
+    g = atlas.get_graph(M, sigma, role)
+    print(f"step case {role} M={M}", flush=True)
+    atlas.replay(g, tokens, positions, cache_len, n_pend=n_pend)
+    toks, conf, accept = atlas.read_outputs(g)
+    rows = g.logits_end - g.logits_start
+    got = atlas.workspace.logits[:rows, : model.args.vocab_size].float().cpu().numpy()
+
+    desc = runtime.step_descriptor(role, M, atlas.D, cache_len, n_pend)
+    vis = runtime.dense_visibility(desc, M, sigma)
+    kk, vv = kv_bits[0].copy(), kv_bits[1].copy()
+    want_bits = DO.decode_step(_oracle_weights(model, atlas), kk, vv, tokens, positions, vis, sigma,
+                               g.logits_start, g.logits_end)
+    from oracle import oracle as O
+    want = O.bf16_bits_to_f32(want_bits)[:, : model.args.vocab_size]
+    tol = 6e-2 * np.abs(want).max()
+    assert np.abs(got - want).max() <= tol
+    # the KV rows the step wrote agree with the oracle's to the last place or two
+    new_k = bf16_bits(atlas.kv(sigma))[0][:, :, sigma:sigma + M]
+    d = np.abs(bf16_ordinal(new_k) - bf16_ordinal(kk[:, :, sigma:sigma + M]))
+    assert np.quantile(d, 0.99) <= 2
+    # argmax / confidence outputs describe the logits the step produced
+    wt, wc, wn = DO.draft_chain(got, atlas.threshold)
+    assert toks.tolist() == wt.tolist()
+    np.testing.assert_allclose(conf, wc, rtol=2e-3, atol=1e-6)
+    assert accept == wn
+
+
+def test_graph_replay_equals_eager_and_is_repeatable(tiny):
+    from bitmtp_amd.runtime import GraphAtlas
+    model, atlas = tiny
+    eager = GraphAtlas(model, segment_ladder=(64, 256), use_graphs=False)
+    rng = np.random.default_rng(5)
+    sigma, cache_len, M = 64, 30, 9
+    hist = _rand_bf16(rng, tuple(atlas.kv(sigma).shape), 0.5).to(DEV)
+    tokens = rng.integers(0, 1000, M).tolist()
+    positions = [cache_len - 1 + i for i in range(M)]
+    outs = []
+    for a in (atlas, eager, atlas, atlas):
+        a.kv(sigma).copy_(hist)
+        g = a.get_graph(M, sigma, "verify")
+        a.replay(g, tokens, positions, cache_len)
+        a.read_outputs(g)
+        outs.append(a.workspace.logits[:M].clone())
+        torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
+def test_wide_causal_replay_matches_sequential_width_one(tiny):
+    """Width-M AR-causal replay == M width-1 replays on the same tokens, within the
+    accumulation-order differences of the two GEMV kernels."""
+    model, atlas = tiny
+    sigma, M = 64, 16
+    rng = np.random.default_rng(9)
+    tokens = rng.integers(0, 1000, M).tolist()
+    atlas.kv(sigma).zero_()
+    gw = atlas.get_graph(M, sigma, "ar")
+    atlas.replay(gw, tokens, list(range(M)), 0)
+    atlas.read_outputs(gw)
+    wide = atlas.workspace.logits[:M, :1000].float().cpu().numpy()
+    atlas.kv(sigma).zero_()
+    g1 = atlas.get_graph(1, sigma, "ar")
+    seq = []
+    for i, t in enumerate(tokens):
+        atlas.replay(g1, [t], [i], i)
+        atlas.commit_kv(sigma, i, 1)
+        atlas.read_outputs(g1)
+        seq.append(atlas.workspace.logits[0, :1000].float().cpu().numpy())
+    seq = np.stack(seq)
+    assert np.abs(wide - seq).max() <= 6e-2 * np.abs(seq).max()
+
+
+def test_hybrid_with_exact_verification_reproduces_ar(tiny):
+    from bitmtp_amd import generate
+    model, atlas = tiny
+    rng = np.random.default_rng(21)
+    prompt = rng.integers(0, 1000, 37).tolist()
+    ar, st_ar = generate.ar_generate(atlas, prompt, max_gen_len=40)
+    hy, st = generate.hybrid_generate(atlas, prompt, max_gen_len=40, exact_m1_verify=True)
+    assert len(ar) == 40 and st_ar["timed_decode_tokens"] == 39
+    assert hy == ar
+    assert st["draft_iters"] == st["n_conf_path"] + st["n_verify_path"]
+    assert st["decode_tokens"] == 1 + st["accepted_drafts"] + st["verifier_bonus_tokens"]
+
+
+@pytest.mark.parametrize("threshold,hybrid_m", [(0.9, None), (0.0, 1), (0.0, 8)])
+def test_hybrid_accounting_and_width_schedule(tiny, threshold, hybrid_m):
+    from bitmtp_amd import generate
+    model, atlas = tiny
+    rng = np.random.default_rng(22)
+    prompt = rng.integers(0, 1000, 50).tolist()
+    before = set(atlas.graphs)
+    out, st = generate.hybrid_generate(atlas, prompt, threshold=threshold, hybrid_m=hybrid_m,
+                                       max_gen_len=64)
+    assert len(out) == 64 and all(0 <= t < 1000 for t in out)
+    assert st["n_iters"] == st["draft_iters"] + 1
+    assert st["drafted_tokens"] == 8 * st["draft_iters"]
+    assert st["committed_tokens"] == 63 == st["timed_decode_tokens"]
+    if threshold == 0.0:
+        # every confidence passes: whole blocks are committed and re-forwarded as 8 pending rows
+        assert st["n_verify_path"] == 0 and st["committed_per_iter"] > 7
+        assert (16, 64, "draft") in atlas.graphs or (16, 256, "draft") in atlas.graphs
+    else:
+        # near-uniform random logits never pass 0.9: draft(9) + verify(9) every iteration
+        # (the last bonus may be clipped by max_gen_len)
+        assert st["n_conf_path"] == 0
+        assert st["n_verify_path"] - 1 <= st["verifier_bonus_tokens"] <= st["n_verify_path"]
+
+
+def test_eos_stops_generation(tiny):
+    from bitmtp_amd import generate
+    model, atlas = tiny
+    prompt = list(range(3, 30))
+    ar, _ = generate.ar_generate(atlas, prompt, max_gen_len=24)
+    eos = ar[10]
+    first = ar.index(eos)
+    cut, st = generate.ar_generate(atlas, prompt, max_gen_len=24, eos_ids=[eos])
+    assert cut == ar[:first]
+    hy, _ = generate.hybrid_generate(atlas, prompt, max_gen_len=24, eos_ids=[eos],
+                                     exact_m1_verify=True)
+    assert hy == ar[:first]
