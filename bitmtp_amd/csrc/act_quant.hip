@@ -118,10 +118,10 @@ __global__ void __launch_bounds__(kThreads) act_quant_kernel(const void *x, int8
 //   normed = bf16( w * bf16(fp32(h) * rs) )           (two bf16 roundings)
 //   s, q   = per-token absmax quantisation of fp32(normed)
 // The sum of squares is accumulated in fp64 in a fixed order (thread-strided, then
-// an xor butterfly per wave, then the four waves left to right), which the CPU
+// an xor butterfly per wave, then the waves left to right), which the CPU
 // oracle replays, so q and s are reproducible bit for bit.
-// One workgroup per token; the row is re-read from L2 instead of being kept in
-// registers (M is at most a few dozen tokens).
+// One workgroup per token; the row is read once and kept in registers, so the kernel
+// is one memory round trip plus two workgroup reductions long.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
@@ -142,15 +142,29 @@ __device__ __forceinline__ void load8_bf16(const uint16_t *row, int v, float out
     }
 }
 
+// Block geometry of the fused producers: one workgroup per token, one 8-element vector
+// per thread and pass, `producer_threads(K/8)` threads, so that a row of up to 8192
+// elements is read from memory exactly once and kept in registers across the two
+// reductions.  Longer rows take several vectors per thread (VPT, a power of two).
+constexpr int kMaxProducerThreads = 1024;
+constexpr int kMaxProducerWaves = kMaxProducerThreads / 64;
+
+__host__ __device__ inline int producer_threads(int nvec) {
+    const int t = ((nvec < kMaxProducerThreads ? nvec : kMaxProducerThreads) + 63) / 64 * 64;
+    return t < 64 ? 64 : t;
+}
+
+// Fixed reduction order (the CPU oracle replays it): thread t accumulates its vectors
+// t, t+T, ... in turn, an xor butterfly (32,16,...,1) inside each wave, then the wave
+// totals left to right.
 __device__ __forceinline__ double block_sum_f64(double v, double *scratch) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
     if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
     __syncthreads();
+    const int waves = blockDim.x >> 6;
     double t = scratch[0];
-#pragma unroll
-    for (int w = 1; w < kThreads / 64; ++w) t += scratch[w];
-    __syncthreads();
+    for (int w = 1; w < waves; ++w) t += scratch[w];
     return t;
 }
 
@@ -159,10 +173,9 @@ __device__ __forceinline__ float block_max_f32(float v, float *scratch) {
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
     if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
     __syncthreads();
+    const int waves = blockDim.x >> 6;
     float t = scratch[0];
-#pragma unroll
-    for (int w = 1; w < kThreads / 64; ++w) t = fmaxf(t, scratch[w]);
-    __syncthreads();
+    for (int w = 1; w < waves; ++w) t = fmaxf(t, scratch[w]);
     return t;
 }
 
@@ -175,114 +188,162 @@ __device__ __forceinline__ void store_q8(int8_t *qrow, int v, const float nf[8],
     reinterpret_cast<uint2 *>(qrow)[v] = o;
 }
 
-template <bool ADD>
-__global__ void __launch_bounds__(kThreads)
+__device__ __forceinline__ void unpack8_bf16(const uint4 raw, float out[8]) {
+    const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[2 * i] = bf16_bits_to_f32(d[i] & 0xffffu);
+        out[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+    }
+}
+
+template <bool ADD, int VPT>
+__global__ void __launch_bounds__(kMaxProducerThreads)
 rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t *w, float eps,
                      uint16_t *h_out, int8_t *q, float *s, int K) {
-    __shared__ double sum_scratch[kThreads / 64];
-    __shared__ float max_scratch[kThreads / 64];
+    __shared__ double sum_scratch[kMaxProducerWaves];
+    __shared__ float max_scratch[kMaxProducerWaves];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
+    const int T = blockDim.x;
     const int nvec = K / 8;
-    const uint16_t *xrow = x + (size_t)m * K;
-    const uint16_t *rrow = ADD ? residual + (size_t)m * K : nullptr;
+    const uint4 *xrow = reinterpret_cast<const uint4 *>(x + (size_t)m * K);
+    const uint4 *rrow = ADD ? reinterpret_cast<const uint4 *>(residual + (size_t)m * K) : nullptr;
+    const uint4 *wrow = reinterpret_cast<const uint4 *>(w);
 
-    auto load_h = [&](int v, float h[8]) {
-        load8_bf16(xrow, v, h);
+    // every load of the row is issued before anything waits on one
+    uint4 xr[VPT], rr[VPT], wr[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * T;
+        const int vc = v < nvec ? v : 0;
+        xr[i] = xrow[vc];
+        if (ADD) rr[i] = rrow[vc];
+        wr[i] = wrow[vc];
+    }
+    float h[VPT][8];
+    double ss = 0.0;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * T;
+        unpack8_bf16(xr[i], h[i]);
         if (ADD) {
             float r[8];
-            load8_bf16(rrow, v, r);
+            unpack8_bf16(rr[i], r);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) h[i] = bf16_round(h[i] + r[i]);
+            for (int e = 0; e < 8; ++e) h[i][e] = bf16_round(h[i][e] + r[e]);
+            if (v < nvec) {
+                uint4 o;
+                o.x = f32_to_bf16_bits(h[i][0]) | (f32_to_bf16_bits(h[i][1]) << 16);
+                o.y = f32_to_bf16_bits(h[i][2]) | (f32_to_bf16_bits(h[i][3]) << 16);
+                o.z = f32_to_bf16_bits(h[i][4]) | (f32_to_bf16_bits(h[i][5]) << 16);
+                o.w = f32_to_bf16_bits(h[i][6]) | (f32_to_bf16_bits(h[i][7]) << 16);
+                reinterpret_cast<uint4 *>(h_out + (size_t)m * K)[v] = o;
+            }
         }
-    };
-
-    double ss = 0.0;
-    for (int v = tid; v < nvec; v += kThreads) {
-        float h[8];
-        load_h(v, h);
-        if (ADD) {
-            uint4 o;
-            o.x = f32_to_bf16_bits(h[0]) | (f32_to_bf16_bits(h[1]) << 16);
-            o.y = f32_to_bf16_bits(h[2]) | (f32_to_bf16_bits(h[3]) << 16);
-            o.z = f32_to_bf16_bits(h[4]) | (f32_to_bf16_bits(h[5]) << 16);
-            o.w = f32_to_bf16_bits(h[6]) | (f32_to_bf16_bits(h[7]) << 16);
-            reinterpret_cast<uint4 *>(h_out + (size_t)m * K)[v] = o;
-        }
+        if (v < nvec) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float sq = h[i] * h[i];
-            ss += (double)sq;
+            for (int e = 0; e < 8; ++e) {
+                const float sq = h[i][e] * h[i][e];
+                ss += (double)sq;
+            }
         }
     }
     const double total = block_sum_f64(ss, sum_scratch);
     const float var = (float)total / (float)K;
     const float rs = 1.0f / sqrtf(var + eps);
 
-    auto normed = [&](int v, float nf[8]) {
-        float h[8], wv[8];
-        load_h(v, h);
-        load8_bf16(w, v, wv);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) nf[i] = bf16_round(wv[i] * bf16_round(h[i] * rs));
-    };
-
     float amax = 0.0f;
-    for (int v = tid; v < nvec; v += kThreads) {
-        float nf[8];
-        normed(v, nf);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(nf[i]));
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * T;
+        float wv[8];
+        unpack8_bf16(wr[i], wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            h[i][e] = bf16_round(wv[e] * bf16_round(h[i][e] * rs));
+            if (v < nvec) amax = fmaxf(amax, fabsf(h[i][e]));
+        }
     }
     amax = block_max_f32(amax, max_scratch);
     const float recip = 1.0f / fmaxf(amax, 1e-5f);
     const float sval = recip * 127.0f;
     if (tid == 0) s[m] = sval;
-
     int8_t *qrow = q + (size_t)m * K;
-    for (int v = tid; v < nvec; v += kThreads) {
-        float nf[8];
-        normed(v, nf);
-        store_q8(qrow, v, nf, sval);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * T;
+        if (v < nvec) store_q8(qrow, v, h[i], sval);
     }
 }
 
 // inner = bf16( fp32(bf16(silu(gate))) * up ), gate = gu[m][0..F), up = gu[m][F..2F)
-__global__ void __launch_bounds__(kThreads)
+template <int VPT>
+__global__ void __launch_bounds__(kMaxProducerThreads)
 silu_mul_quant_kernel(const uint16_t *gu, int8_t *q, float *s, int F) {
-    __shared__ float max_scratch[kThreads / 64];
+    __shared__ float max_scratch[kMaxProducerWaves];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
+    const int T = blockDim.x;
     const int nvec = F / 8;
-    const uint16_t *grow = gu + (size_t)m * 2 * F;
-    const uint16_t *urow = grow + F;
-
-    auto inner = [&](int v, float nf[8]) {
-        float g[8], u[8];
-        load8_bf16(grow, v, g);
-        load8_bf16(urow, v, u);
+    const uint4 *grow = reinterpret_cast<const uint4 *>(gu + (size_t)m * 2 * F);
+    const uint4 *urow = reinterpret_cast<const uint4 *>(gu + (size_t)m * 2 * F + F);
+    uint4 gr[VPT], ur[VPT];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float sg = bf16_round(g[i] / (1.0f + expf(-g[i])));
-            nf[i] = bf16_round(sg * u[i]);
-        }
-    };
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * T;
+        const int vc = v < nvec ? v : 0;
+        gr[i] = grow[vc];
+        ur[i] = urow[vc];
+    }
+    float nf[VPT][8];
     float amax = 0.0f;
-    for (int v = tid; v < nvec; v += kThreads) {
-        float nf[8];
-        inner(v, nf);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(nf[i]));
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * T;
+        float g[8], u[8];
+        unpack8_bf16(gr[i], g);
+        unpack8_bf16(ur[i], u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sg = bf16_round(g[e] / (1.0f + expf(-g[e])));
+            nf[i][e] = bf16_round(sg * u[e]);
+            if (v < nvec) amax = fmaxf(amax, fabsf(nf[i][e]));
+        }
     }
     amax = block_max_f32(amax, max_scratch);
     const float recip = 1.0f / fmaxf(amax, 1e-5f);
     const float sval = recip * 127.0f;
     if (tid == 0) s[m] = sval;
     int8_t *qrow = q + (size_t)m * F;
-    for (int v = tid; v < nvec; v += kThreads) {
-        float nf[8];
-        inner(v, nf);
-        store_q8(qrow, v, nf, sval);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int v = tid + i * T;
+        if (v < nvec) store_q8(qrow, v, nf[i], sval);
+    }
+}
+
+// vectors per thread for a row of nvec 8-element vectors: 1, 2, 4 or 8
+inline int producer_vpt(int nvec) {
+    const int t = producer_threads(nvec);
+    const int need = (nvec + t - 1) / t;
+    int vpt = 1;
+    while (vpt < need) vpt *= 2;
+    return vpt;
+}
+
+constexpr int kMaxProducerK = 8 * kMaxProducerThreads * 8;  // VPT <= 8
+
+template <bool ADD>
+void launch_rmsnorm(const uint16_t *x, const uint16_t *r, const uint16_t *w, float eps,
+                    uint16_t *h_out, int8_t *q, float *s, int M, int K, hipStream_t st) {
+    const int nvec = K / 8;
+    const dim3 grid(M), block(producer_threads(nvec));
+    switch (producer_vpt(nvec)) {
+        case 1: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 1>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
+        case 2: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 2>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
+        case 4: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 4>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
+        default: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 8>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
     }
 }
 
@@ -312,10 +373,10 @@ extern "C" int bonsai_act_quant_int8(const void *x, int x_kind, int8_t *q, float
 extern "C" int bonsai_rmsnorm_quant_int8(const void *x, const void *w, float eps, int8_t *q, float *s,
                                          int M, int K, void *stream) {
     if (x == nullptr || w == nullptr || q == nullptr || s == nullptr) return BONSAI_ERR_ARG;
-    if (M < 1 || K < 8 || K % 8 != 0) return BONSAI_ERR_ARG;
-    hipLaunchKernelGGL(rmsnorm_quant_kernel<false>, dim3(M), dim3(kThreads), 0,
-                       static_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t *>(x),
-                       nullptr, reinterpret_cast<const uint16_t *>(w), eps, nullptr, q, s, K);
+    if (M < 1 || K < 8 || K % 8 != 0 || K > kMaxProducerK) return BONSAI_ERR_ARG;
+    launch_rmsnorm<false>(reinterpret_cast<const uint16_t *>(x), nullptr,
+                          reinterpret_cast<const uint16_t *>(w), eps, nullptr, q, s, M, K,
+                          static_cast<hipStream_t>(stream));
     return hipGetLastError() == hipSuccess ? BONSAI_OK : BONSAI_ERR_LAUNCH;
 }
 
@@ -325,21 +386,28 @@ extern "C" int bonsai_add_rmsnorm_quant_int8(const void *x, const void *residual
     if (x == nullptr || residual == nullptr || w == nullptr || h_out == nullptr || q == nullptr ||
         s == nullptr)
         return BONSAI_ERR_ARG;
-    if (M < 1 || K < 8 || K % 8 != 0) return BONSAI_ERR_ARG;
-    hipLaunchKernelGGL(rmsnorm_quant_kernel<true>, dim3(M), dim3(kThreads), 0,
-                       static_cast<hipStream_t>(stream), reinterpret_cast<const uint16_t *>(x),
-                       reinterpret_cast<const uint16_t *>(residual),
-                       reinterpret_cast<const uint16_t *>(w), eps,
-                       reinterpret_cast<uint16_t *>(h_out), q, s, K);
+    if (M < 1 || K < 8 || K % 8 != 0 || K > kMaxProducerK) return BONSAI_ERR_ARG;
+    launch_rmsnorm<true>(reinterpret_cast<const uint16_t *>(x),
+                         reinterpret_cast<const uint16_t *>(residual),
+                         reinterpret_cast<const uint16_t *>(w), eps,
+                         reinterpret_cast<uint16_t *>(h_out), q, s, M, K,
+                         static_cast<hipStream_t>(stream));
     return hipGetLastError() == hipSuccess ? BONSAI_OK : BONSAI_ERR_LAUNCH;
 }
 
 extern "C" int bonsai_silu_mul_quant_int8(const void *gate_up, int8_t *q, float *s, int M, int F,
                                           void *stream) {
     if (gate_up == nullptr || q == nullptr || s == nullptr) return BONSAI_ERR_ARG;
-    if (M < 1 || F < 8 || F % 8 != 0) return BONSAI_ERR_ARG;
-    hipLaunchKernelGGL(silu_mul_quant_kernel, dim3(M), dim3(kThreads), 0,
-                       static_cast<hipStream_t>(stream),
-                       reinterpret_cast<const uint16_t *>(gate_up), q, s, F);
+    if (M < 1 || F < 8 || F % 8 != 0 || F > kMaxProducerK) return BONSAI_ERR_ARG;
+    const int nvec = F / 8;
+    const dim3 grid(M), block(producer_threads(nvec));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t *gu = reinterpret_cast<const uint16_t *>(gate_up);
+    switch (producer_vpt(nvec)) {
+        case 1: hipLaunchKernelGGL(silu_mul_quant_kernel<1>, grid, block, 0, st, gu, q, s, F); break;
+        case 2: hipLaunchKernelGGL(silu_mul_quant_kernel<2>, grid, block, 0, st, gu, q, s, F); break;
+        case 4: hipLaunchKernelGGL(silu_mul_quant_kernel<4>, grid, block, 0, st, gu, q, s, F); break;
+        default: hipLaunchKernelGGL(silu_mul_quant_kernel<8>, grid, block, 0, st, gu, q, s, F); break;
+    }
     return hipGetLastError() == hipSuccess ? BONSAI_OK : BONSAI_ERR_LAUNCH;
 }

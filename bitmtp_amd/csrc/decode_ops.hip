@@ -142,7 +142,7 @@ struct AttnArgs {
 
 template <int RW>
 __global__ void __launch_bounds__(64) attn_partial_kernel(AttnArgs a) {
-    __shared__ float p_lds[RW][kChunk];
+    __shared__ __attribute__((aligned(16))) float p_lds[RW][kChunk];
     const int lane = threadIdx.x;
     int id = blockIdx.x;
     const int kvh = id % a.n_kv;
@@ -170,6 +170,16 @@ __global__ void __launch_bounds__(64) attn_partial_kernel(AttnArgs a) {
     uint4 kreg[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) kreg[i] = krow[i];
+    // the V rows of the chunk (lane = 2 dims) are requested now as well, so that the
+    // kernel is one memory round trip long; rows past the live part repeat the last one
+    const uint32_t *vbase = a.v_layer + (size_t)kvh * a.slots * 64 + lane;
+    uint32_t vreg[kChunk];
+#pragma unroll
+    for (int j = 0; j < kChunk; ++j) {
+        const int tj = min(t0 + j, total - 1);
+        const int sj = tj < cache_len ? tj : a.sigma + (tj - cache_len);
+        vreg[j] = vbase[(size_t)sj * 64];
+    }
 
     const int row0 = rg * RW;
     float mrow[RW], lrow[RW];
@@ -198,32 +208,26 @@ __global__ void __launch_bounds__(64) attn_partial_kernel(AttnArgs a) {
         const float p = (mx == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(sc - mx);
         mrow[r] = mx;
         lrow[r] = wave_sum(p);
-        p_lds[r][lane] = p;
+        p_lds[r][lane] = p;   // dead lanes hold 0
     }
     __syncthreads();
 
-    // ---- phase 2: acc[r][2 dims] over the live slots of the chunk
+    // ---- phase 2: acc[r][2 dims] over the slots of the chunk (p is 0 for dead slots)
     float acc[RW][2];
 #pragma unroll
     for (int r = 0; r < RW; ++r) acc[r][0] = acc[r][1] = 0.0f;
-    const uint32_t *vbase = a.v_layer + (size_t)kvh * a.slots * 64 + lane;
-    constexpr int UN = 8;
-    for (int j0 = 0; j0 < n_live; j0 += UN) {
-        uint32_t vv[UN];
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int tj = min(t0 + j0 + u, total - 1);
-            const int sj = tj < cache_len ? tj : a.sigma + (tj - cache_len);
-            vv[u] = vbase[(size_t)sj * 64];
-        }
+    for (int j = 0; j < kChunk; j += 4) {
+        float4 pj[RW];
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const float v0 = bf16_bits_to_f32(vv[u] & 0xffffu);
-            const float v1 = __uint_as_float(vv[u] & 0xffff0000u);
-            const bool in = (j0 + u) < n_live;
+        for (int r = 0; r < RW; ++r) pj[r] = *reinterpret_cast<const float4 *>(&p_lds[r][j]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float v0 = bf16_bits_to_f32(vreg[j + u] & 0xffffu);
+            const float v1 = __uint_as_float(vreg[j + u] & 0xffff0000u);
 #pragma unroll
             for (int r = 0; r < RW; ++r) {
-                const float p = in ? p_lds[r][j0 + u] : 0.0f;
+                const float p = u == 0 ? pj[r].x : (u == 1 ? pj[r].y : (u == 2 ? pj[r].z : pj[r].w));
                 acc[r][0] = fmaf(p, v0, acc[r][0]);
                 acc[r][1] = fmaf(p, v1, acc[r][1]);
             }
@@ -255,15 +259,47 @@ struct CombineArgs {
 };
 
 constexpr int kCombineThreads = 256;
-constexpr int kCombineMaxVec = 2;  // 8-element vectors per thread: up to 32 heads
+constexpr int kCombineMaxVec = 2;      // 8-element vectors per thread: up to 32 heads
+constexpr int kCombineMaxHeads = kCombineThreads * kCombineMaxVec / (kHd / 8);
+constexpr int kCombineMaxChunks = 136;  // sigma + M up to 8704 slots
 
 __global__ void __launch_bounds__(kCombineThreads) attn_combine_kernel(CombineArgs a) {
+    __shared__ float wgt[kCombineMaxHeads * kCombineMaxChunks];  // becomes the chunk weights
+    __shared__ float lsum[kCombineMaxHeads * kCombineMaxChunks];
     __shared__ float max_scratch[kCombineThreads / 64];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
     const int total = min(max(a.meta[0], 0), a.sigma) + a.M;
     const int live_chunks = (total + kChunk - 1) / kChunk;
     const int nvec = a.n_heads * (kHd / 8);
+    const float *row = a.part + (size_t)m * a.n_heads * a.n_chunks * kPartStride;
+
+    // (max, sum) of every (head, chunk): one load per thread and pass
+    const int pairs = a.n_heads * live_chunks;
+    for (int idx = tid; idx < pairs; idx += kCombineThreads) {
+        const int head = idx / live_chunks, c = idx % live_chunks;
+        const float2 ml = *reinterpret_cast<const float2 *>(
+            row + ((size_t)head * a.n_chunks + c) * kPartStride + kHd);
+        wgt[idx] = ml.x;
+        lsum[idx] = ml.y;
+    }
+    __syncthreads();
+    if (tid < a.n_heads) {  // one thread per head turns them into normalised chunk weights
+        float *wh = wgt + tid * live_chunks;
+        const float *lh = lsum + tid * live_chunks;
+        float mx = -INFINITY;
+        for (int c = 0; c < live_chunks; ++c) mx = fmaxf(mx, wh[c]);
+        float den = 0.0f;
+        for (int c = 0; c < live_chunks; ++c) {
+            const float e = (wh[c] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(wh[c] - mx);
+            wh[c] = e;
+            den = fmaf(e, lh[c], den);
+        }
+        const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+        for (int c = 0; c < live_chunks; ++c) wh[c] *= inv;
+    }
+    __syncthreads();
+
     float o[kCombineMaxVec][8];
     float amax = 0.0f;
 #pragma unroll
@@ -274,32 +310,24 @@ __global__ void __launch_bounds__(kCombineThreads) attn_combine_kernel(CombineAr
         if (v >= nvec) continue;
         const int head = v / (kHd / 8);
         const int d0 = (v % (kHd / 8)) * 8;
-        const float *base = a.part + ((size_t)m * a.n_heads + head) * a.n_chunks * kPartStride;
-        float mx = -INFINITY;
-        for (int c = 0; c < live_chunks; ++c) mx = fmaxf(mx, base[(size_t)c * kPartStride + kHd]);
-        float den = 0.0f;
+        const float *base = row + (size_t)head * a.n_chunks * kPartStride + d0;
+        const float *wh = wgt + head * live_chunks;
         float num[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) num[i] = 0.0f;
-        if (mx != -INFINITY) {
-            for (int c = 0; c < live_chunks; ++c) {
-                const float *pc = base + (size_t)c * kPartStride;
-                const float mc = pc[kHd];
-                if (mc == -INFINITY) continue;
-                const float wgt = __builtin_amdgcn_exp2f(mc - mx);
-                den = fmaf(wgt, pc[kHd + 1], den);
-                const float4 x0 = reinterpret_cast<const float4 *>(pc + d0)[0];
-                const float4 x1 = reinterpret_cast<const float4 *>(pc + d0)[1];
-                num[0] = fmaf(wgt, x0.x, num[0]); num[1] = fmaf(wgt, x0.y, num[1]);
-                num[2] = fmaf(wgt, x0.z, num[2]); num[3] = fmaf(wgt, x0.w, num[3]);
-                num[4] = fmaf(wgt, x1.x, num[4]); num[5] = fmaf(wgt, x1.y, num[5]);
-                num[6] = fmaf(wgt, x1.z, num[6]); num[7] = fmaf(wgt, x1.w, num[7]);
-            }
+#pragma unroll 4
+        for (int c = 0; c < live_chunks; ++c) {
+            const float4 x0 = reinterpret_cast<const float4 *>(base + (size_t)c * kPartStride)[0];
+            const float4 x1 = reinterpret_cast<const float4 *>(base + (size_t)c * kPartStride)[1];
+            const float w = wh[c];
+            num[0] = fmaf(w, x0.x, num[0]); num[1] = fmaf(w, x0.y, num[1]);
+            num[2] = fmaf(w, x0.z, num[2]); num[3] = fmaf(w, x0.w, num[3]);
+            num[4] = fmaf(w, x1.x, num[4]); num[5] = fmaf(w, x1.y, num[5]);
+            num[6] = fmaf(w, x1.z, num[6]); num[7] = fmaf(w, x1.w, num[7]);
         }
-        const float inv = den > 0.0f ? 1.0f / den : 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            o[it][i] = bf16_round(num[i] * inv);
+            o[it][i] = bf16_round(num[i]);
             amax = fmaxf(amax, fabsf(o[it][i]));
         }
         if (a.out_bf16 != nullptr) {
@@ -508,7 +536,8 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
     if ((out_q == nullptr) != (out_s == nullptr)) return BONSAI_DECODE_ERR_ARG;
     if (!out_bf16 && !out_q) return BONSAI_DECODE_ERR_ARG;
     if (M < 1 || M > BONSAI_MAX_WIDTH || n_kv < 1 || n_heads < n_kv || n_heads % n_kv != 0 ||
-        n_heads > kCombineThreads * kCombineMaxVec / (kHd / 8) || sigma < 0 || sigma + M > slots)
+        n_heads > kCombineMaxHeads || sigma < 0 || sigma + M > slots ||
+        (sigma + M + kChunk - 1) / kChunk > kCombineMaxChunks)
         return BONSAI_DECODE_ERR_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     AttnArgs a;

@@ -264,15 +264,18 @@ void oracle_gemv(const int8_t *A, const uint8_t *B, const float *S, const uint16
 
 static inline float bf16_round_f(float f) { return oracle_bf16_to_f32(oracle_f32_to_bf16(f)); }
 
-/* Sum of fp32 squares in fp64, in the order the HIP kernel uses: 256 threads, thread t
- * takes the 8-element vectors t, t+256, ... in turn; xor butterfly (32,16,..,1) inside
- * each 64-thread wave; the four wave totals added left to right. */
+/* Sum of fp32 squares in fp64, in the order the HIP kernel uses: T threads with
+ * T = min(1024, K/8 rounded up to a multiple of 64); thread t takes the 8-element
+ * vectors t, t+T, ... in turn; xor butterfly (32,16,..,1) inside each 64-thread wave;
+ * the wave totals added left to right. */
 static double sumsq_kernel_order(const float *h, int K) {
-    double lane[256];
+    static double lane[1024];
     int nvec = K / 8;
-    for (int t = 0; t < 256; ++t) {
+    int T = ((nvec < 1024 ? nvec : 1024) + 63) / 64 * 64;
+    if (T < 64) T = 64;
+    for (int t = 0; t < T; ++t) {
         double acc = 0.0;
-        for (int v = t; v < nvec; v += 256)
+        for (int v = t; v < nvec; v += T)
             for (int i = 0; i < 8; ++i) {
                 volatile float sq = h[8 * v + i] * h[8 * v + i];
                 acc += (double)sq;
@@ -280,7 +283,7 @@ static double sumsq_kernel_order(const float *h, int K) {
         lane[t] = acc;
     }
     double total = 0.0;
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < T / 64; ++w) {
         double a[64], b[64];
         for (int i = 0; i < 64; ++i) a[i] = lane[64 * w + i];
         for (int off = 32; off > 0; off >>= 1) {
