@@ -63,11 +63,11 @@ int launch_matrix_core(bool fp4, bool single_tile, const int8_t *A, const uint8_
     int ks = tu.k_split;
     int R = tu.row_tiles;
     const int ntiles = K / 512;
-    if (ks == 0)
-        ks = (ntiles % 4 == 0 && (long)N * 4 <= 16384) ? 4
-             : ((ntiles % 2 == 0 && (long)N * 2 <= 16384) ? 2 : 1);
+    if (ks == 0) ks = (N <= 4096 && ntiles >= 4) ? 4 : ((N <= 16384 && ntiles >= 2) ? 2 : 1);
     if (ks != 1 && ks != 2 && ks != 4) ks = 1;
-    if (ks > ntiles || ntiles % ks != 0) ks = 1;  // equal K slices: the waves meet at one barrier
+    // slices may be uneven (tile t goes to slice floor-partition): every wave still reaches the
+    // single barrier after its K loop; an empty slice is never scheduled
+    if (ks > ntiles) ks = 1;
     if (R == 0) {
         const long wgs1 = ((long)N + 16 * (4 / ks) - 1) / (16 * (4 / ks));  // workgroups at R = 1
         R = wgs1 >= 8192 ? 4 : (wgs1 >= 2048 ? 2 : 1);
