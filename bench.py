@@ -170,6 +170,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--layers", type=int, default=48, help="distinct layers in the weight pool")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--no-decode", action="store_true",
+                    help="skip the end-to-end decode tokens/s section")
     ap.add_argument("--no-head", action="store_true", help="skip the lm_head-sized extra measurement")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device copy (for scaling rocprofv3 PMC byte counters)")
@@ -271,6 +273,15 @@ def main() -> int:
         dst.copy_(src)
         torch.cuda.synchronize()
 
+    # The other half of the headline metric: end-to-end decode tokens/s of the random-init
+    # 1.7B-shaped model (configs[2]), AR and D8 hybrid, by the reference's timing contract.
+    decode = None
+    if not args.no_decode:
+        del run, pool, graph
+        torch.cuda.empty_cache()
+        from bitmtp_amd.decode_bench import run_decode_bench
+        decode = run_decode_bench("1.7b", prompt_len=256, new_tokens=512, repeats=1)
+
     cpu = cpu_baseline(args.cpu_seconds) if args.cpu_seconds > 0 else None
 
     line = {
@@ -287,6 +298,7 @@ def main() -> int:
             "per_width": {str(m): per_width[m] for m in WIDTHS},
             "timing": "one HIP graph of all steps, HIP events on the launch stream, best of 3 replays",
             "lm_head_151936x2048": head,
+            "decode_1p7b_d8": decode,
         },
         "roofline": roofline,
         "cpu_baseline": cpu,
