@@ -237,7 +237,7 @@ def main() -> int:
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "traffic": round(MEASURED_TRAFFIC_BYTES[dom]),
-        "kernel": (f"gemv_mfma_kernel<BITS=2> (width {dom})" if dom >= 5
+        "kernel": (f"gemv_mfma_direct_kernel<BITS=2> (width {dom})" if dom >= 3
                    else f"gemv_dot4_kernel<BITS=2, MT={dom}> (width {dom})"),
         "bytes_per_launch": round(bytes_per_launch),
         "us_per_launch": per_width[dom]["us_per_launch"],

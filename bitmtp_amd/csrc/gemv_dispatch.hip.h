@@ -18,7 +18,8 @@
 
 namespace bonsai {
 
-constexpr int kDefaultMfmaMinWidth = 5;       // layer-sized matrices
+constexpr int kDefaultMfmaMinWidth = 3;       // layer-sized matrices (dot4 wins at 1 and 2 tokens)
+constexpr int kDirectMaxRows = 16384;         // up to here the staging-free matrix-core kernel
 constexpr int kLongMatrixRows = 32768;        // from here on the matrix cores pay off at M >= 2
 
 template <int BITS>
@@ -43,12 +44,14 @@ int init_all_kernels() {
 // refuses shapes whose tokens would need more than ceil(M/16) token tiles, i.e.
 // a second pass over the weights.
 template <int BITS>
-int launch_matrix_core(bool fp4, bool single_tile, const int8_t *A, const uint8_t *B, void *out,
+int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint8_t *B, void *out,
                        const float *s, const void *ws, int M, int N, int K, int out_kind,
                        int scale_kind, int lds_limit, hipStream_t stream) {
     const MfmaTuning &tu = mfma_tuning<BITS>();
+    const bool fp4 = engine == 2, direct = engine == 3;
     auto lds_for = [&](int ri, int mt) {
-        return fp4 ? fp4_lds_for<BITS>(ri, mt, K) : mfma_lds_for<BITS>(ri, mt, K);
+        return fp4 ? fp4_lds_for<BITS>(ri, mt, K)
+                   : (direct ? mfma_direct_lds_for<BITS>(ri) : mfma_lds_for<BITS>(ri, mt, K));
     };
     int ntok_tiles = (M + kMfmaTokens - 1) / kMfmaTokens;
     int mt = (M + ntok_tiles - 1) / ntok_tiles;
@@ -63,7 +66,12 @@ int launch_matrix_core(bool fp4, bool single_tile, const int8_t *A, const uint8_
     int ks = tu.k_split;
     int R = tu.row_tiles;
     const int ntiles = K / 512;
-    if (ks == 0) ks = (N <= 4096 && ntiles >= 4) ? 4 : ((N <= 16384 && ntiles >= 2) ? 2 : 1);
+    if (ks == 0) {
+        if (direct)  // no staging to amortise: split K as far as it goes
+            ks = ntiles >= 4 ? 4 : (ntiles >= 2 ? 2 : 1);
+        else
+            ks = (N <= 4096 && ntiles >= 4) ? 4 : ((N <= 16384 && ntiles >= 2) ? 2 : 1);
+    }
     if (ks != 1 && ks != 2 && ks != 4) ks = 1;
     // slices may be uneven (tile t goes to slice floor-partition): every wave still reaches the
     // single barrier after its K loop; an empty slice is never scheduled
@@ -105,7 +113,9 @@ int launch_matrix_core(bool fp4, bool single_tile, const int8_t *A, const uint8_
     const int rows_per_wg = 16 * R * (4 / ks) * passes;
     const int grid_x = (N + rows_per_wg - 1) / rows_per_wg;
     const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
-    const MfmaKernelFn fn = fp4 ? fp4_table<BITS>().fn[ri][variant] : mfma_table<BITS>().fn[ri][variant];
+    const MfmaKernelFn fn = fp4 ? fp4_table<BITS>().fn[ri][variant]
+                                : (direct ? mfma_direct_table<BITS>().fn[ri][variant]
+                                          : mfma_table<BITS>().fn[ri][variant]);
     hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(kMfmaThreads, 1, 1), lds_for(ri, mt),
                        stream, args);
     return hipGetLastError() == hipSuccess ? 0 : 2;
@@ -134,11 +144,13 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
                                             : (N >= kLongMatrixRows ? 2 : kDefaultMfmaMinWidth);
     if (M >= min_width && mfma_shape_ok(B, out_kind == OUT_G32 ? nullptr : ws, K)) {
         int rc = -1;
-        if (mtu.engine == 2)
-            rc = launch_matrix_core<BITS>(true, false, A, B, out, s, ws, M, N, K, out_kind,
+        // operand-loaded activations win up to about 16k rows, staged ones above (measured)
+        const int engine = mtu.engine != 0 ? mtu.engine : (N <= kDirectMaxRows ? 3 : 1);
+        if (engine == 2 || engine == 3)
+            rc = launch_matrix_core<BITS>(engine, false, A, B, out, s, ws, M, N, K, out_kind,
                                           scale_kind, lds_limit, stream);
         if (rc < 0)
-            rc = launch_matrix_core<BITS>(false, false, A, B, out, s, ws, M, N, K, out_kind,
+            rc = launch_matrix_core<BITS>(1, false, A, B, out, s, ws, M, N, K, out_kind,
                                           scale_kind, lds_limit, stream);
         if (rc >= 0) return rc;
     }

@@ -304,6 +304,235 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel(const MfmaArgs 
 }
 
 // ---------------------------------------------------------------------------
+// Same contraction without the activation staging pass: every wave loads the A operand of
+// its K tiles straight from the row-major activations (lane = token, K-block: 32 contiguous
+// bytes per group, an L2 hit) together with the weight tile, permutes them in registers to
+// the order the unpack produces, and obtains the offset-removal terms from two more MFMAs
+// against an all-ones operand (sum of a token's activations over the group, delivered in
+// the accumulator layout).  No workgroup barrier before the K loop and no LDS for
+// activations: the kernel is one memory round trip plus the K loop long.
+// ---------------------------------------------------------------------------
+template <int BITS, int R>
+__host__ __device__ inline size_t mfma_direct_lds_bytes() {
+    return (size_t)4 * mfma_wave_tile_bytes<BITS, R>() + (size_t)4 * R * 4 * 64 * 4;
+}
+
+template <int BITS, int R, bool G32, bool SF16>
+__global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_direct_kernel(const MfmaArgs a) {
+    using MF = MfmaFmt<BITS>;
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int K = a.K, N = a.N, M = a.M;
+    const int G = K / kGroup;
+    const int row_bytes = K * BITS / 8;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int ks = 1 << a.ks_log2;
+    const int kslice = wave & (ks - 1);
+    const int rw = wave >> a.ks_log2;
+    const int rws = 4 >> a.ks_log2;
+    const int m0 = blockIdx.y * a.mt;
+    const int mt = (M - m0) < a.mt ? (M - m0) : a.mt;
+    const int pass_rows = rws * 16 * R;
+    const int n_first = (int)blockIdx.x * a.passes * pass_rows + rw * (16 * R);
+
+    unsigned char *tiles = smem;
+    unsigned char *wt = tiles + (size_t)wave * mfma_wave_tile_bytes<BITS, R>();
+    float *red = reinterpret_cast<float *>(tiles + (size_t)4 * mfma_wave_tile_bytes<BITS, R>());
+
+    const int ntiles = G / kMfmaGroupsPerTile;
+    const int t_begin = (int)(((long)ntiles * kslice) >> a.ks_log2);
+    const int t_end = (int)(((long)ntiles * (kslice + 1)) >> a.ks_log2);
+
+    const int ld_row = lane / MF::kLanesPerRow;
+    const int ld_col = lane % MF::kLanesPerRow;
+    const int op_row = lane & 15;
+    const int kb = lane >> 4;
+    const int a_tok = m0 + (op_row < mt ? op_row : mt - 1);  // tokens past the tile alias the last
+    const int8_t *a_lane = a.A + (size_t)a_tok * K + 32 * kb;
+
+    struct TileRegs {
+        u32x4 w[R][MF::kLoads];
+        uint2 sc[R];
+    };
+    struct ActRegs {
+        u32x4 lo[kMfmaGroupsPerTile], hi[kMfmaGroupsPerTile];  // 32 natural-order bytes per group
+    };
+    auto load_tile = [&](TileRegs &tr, int n0, int kt) {
+#pragma unroll
+        for (int rt = 0; rt < R; ++rt) {
+#pragma unroll
+            for (int h = 0; h < MF::kLoads; ++h) {
+                int row = n0 + rt * 16 + h * MF::kRowsPerLoad + ld_row;
+                row = row < N ? row : N - 1;
+                const unsigned char *p =
+                    a.B + (size_t)row * row_bytes + (size_t)kt * MF::kTileBytes + ld_col * 16;
+                tr.w[rt][h] = *reinterpret_cast<const u32x4 *>(p);
+            }
+            if (!G32) {
+                int row = n0 + rt * 16 + op_row;
+                row = row < N ? row : N - 1;
+                tr.sc[rt] = *reinterpret_cast<const uint2 *>(a.ws + (size_t)row * G +
+                                                             (size_t)kt * kMfmaGroupsPerTile);
+            }
+        }
+    };
+    auto load_act = [&](ActRegs &ar, int kt) {
+#pragma unroll
+        for (int gi = 0; gi < kMfmaGroupsPerTile; ++gi) {
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(
+                a_lane + (size_t)(kt * kMfmaGroupsPerTile + gi) * kGroup);
+            ar.lo[gi] = p[0];
+            ar.hi[gi] = p[1];
+        }
+    };
+    auto park_tile = [&](const TileRegs &tr) {
+#pragma unroll
+        for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+            for (int h = 0; h < MF::kLoads; ++h) {
+                unsigned char *dst = wt + (rt * 16 + h * MF::kRowsPerLoad + ld_row) * MF::kPitch +
+                                     ld_col * 16;
+                uint2 *d2 = reinterpret_cast<uint2 *>(dst);
+                d2[0] = make_uint2(tr.w[rt][h].x, tr.w[rt][h].y);
+                d2[1] = make_uint2(tr.w[rt][h].z, tr.w[rt][h].w);
+            }
+    };
+
+    TileRegs cur;
+    ActRegs acur;
+    if (t_begin < t_end) {
+        load_act(acur, t_begin);
+        load_tile(cur, n_first, t_begin);
+    }
+    float sdiv[4];
+    if (!G32) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = m0 + 4 * kb + r;
+            sdiv[r] = a.s[m < M ? m : M - 1];
+        }
+    }
+
+    float acc[R][4];
+#pragma unroll
+    for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[rt][r] = 0.0f;
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    const v4i zero = {0, 0, 0, 0};
+
+    for (int pass = 0; pass < a.passes; ++pass) {
+        const int n0 = n_first + pass * pass_rows;
+        for (int kt = t_begin; kt < t_end; ++kt) {
+            park_tile(cur);
+            TileRegs nxt;
+            ActRegs anxt;
+            const bool last_kt = kt + 1 == t_end;
+            const bool more = !last_kt || pass + 1 < a.passes;
+            if (more) {
+                load_act(anxt, last_kt ? t_begin : kt + 1);
+                load_tile(nxt, last_kt ? n0 + pass_rows : n0, last_kt ? t_begin : kt + 1);
+            }
+#pragma unroll
+            for (int gi = 0; gi < kMfmaGroupsPerTile; ++gi) {
+                const int g = kt * kMfmaGroupsPerTile + gi;
+                u32x4 a0, a1;
+                if (BITS == 2) {
+                    a0 = transpose4x4_bytes(acur.lo[gi].x, acur.lo[gi].y, acur.lo[gi].z, acur.lo[gi].w);
+                    a1 = transpose4x4_bytes(acur.hi[gi].x, acur.hi[gi].y, acur.hi[gi].z, acur.hi[gi].w);
+                } else {
+                    a0 = transpose4x4_bytes(acur.lo[gi].x, acur.lo[gi].z, acur.hi[gi].x, acur.hi[gi].z);
+                    a1 = transpose4x4_bytes(acur.lo[gi].y, acur.lo[gi].w, acur.hi[gi].y, acur.hi[gi].w);
+                }
+                const v4i va0 = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w};
+                const v4i va1 = {(int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                // sum of the group's activations per token, in the accumulator layout
+                v4i asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, ones, zero, 0, 0, 0);
+                asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, ones, asum, 0, 0, 0);
+                const v4i vcr = {mfma_corr<BITS>(asum[0]), mfma_corr<BITS>(asum[1]),
+                                 mfma_corr<BITS>(asum[2]), mfma_corr<BITS>(asum[3])};
+#pragma unroll
+                for (int rt = 0; rt < R; ++rt) {
+                    const unsigned char *src = wt + (rt * 16 + op_row) * MF::kPitch;
+                    uint32_t p0, p1;
+                    if (BITS == 2) {
+                        const uint2 pp = *reinterpret_cast<const uint2 *>(src + gi * 32 + kb * 8);
+                        p0 = pp.x;
+                        p1 = pp.y;
+                    } else {
+                        p0 = *reinterpret_cast<const uint32_t *>(src + gi * 16 + kb * 4);
+                        p1 = 0;
+                    }
+                    uint32_t b0[4], b1[4];
+                    mfma_unpack<BITS>(p0, p1, b0, b1);
+                    const v4i vb0 = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3]};
+                    const v4i vb1 = {(int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+                    v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, vb0, vcr, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, vb1, d, 0, 0, 0);
+                    if (G32) {
+                        const int row = n0 + rt * 16 + op_row;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int tok = 4 * kb + r;
+                            if (row < N && tok < mt)
+                                reinterpret_cast<int32_t *>(
+                                    a.out)[((size_t)(m0 + tok) * N + row) * G + g] = d[r];
+                        }
+                    } else {
+                        const uint32_t raw = (gi & 2) ? cur.sc[rt].y : cur.sc[rt].x;
+                        const float wsf = scale_to_f32<SF16>(
+                            (uint16_t)((gi & 1) ? (raw >> 16) : (raw & 0xffffu)));
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[rt][r] += (float)d[r] * wsf;
+                    }
+                }
+            }
+            if (more) {
+                cur = nxt;
+                acur = anxt;
+            }
+        }
+
+        if (G32) continue;
+        if (ks > 1) {
+            float *mine = red + (size_t)wave * (R * 4 * 64);
+#pragma unroll
+            for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mine[(rt * 4 + r) * 64 + lane] = acc[rt][r];
+            __syncthreads();
+            if (kslice != 0) return;
+            for (int k2 = 1; k2 < ks; ++k2) {
+                const float *other = red + (size_t)(wave + k2) * (R * 4 * 64);
+#pragma unroll
+                for (int rt = 0; rt < R; ++rt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[rt][r] += other[(rt * 4 + r) * 64 + lane];
+            }
+        }
+#pragma unroll
+        for (int rt = 0; rt < R; ++rt) {
+            const int row = n0 + rt * 16 + op_row;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int tok = 4 * kb + r;
+                if (row < N && tok < mt) {
+                    const float y = acc[rt][r] / sdiv[r];
+                    const size_t o = (size_t)(m0 + tok) * N + row;
+                    if (a.out_f32)
+                        reinterpret_cast<float *>(a.out)[o] = y;
+                    else
+                        reinterpret_cast<uint16_t *>(a.out)[o] = f32_to_bf16_rne(y);
+                }
+                acc[rt][r] = 0.0f;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
 struct MfmaTuning {
@@ -311,7 +540,7 @@ struct MfmaTuning {
     int row_tiles = 0;   // R: 1, 2 or 4; 0 = heuristic
     int k_split = 0;     // waves along K: 1, 2 or 4; 0 = heuristic
     int passes = 0;      // row blocks per workgroup; 0 = heuristic
-    int engine = 0;      // 0 = choose, 1 = int8 MFMA only, 2 = FP4 x FP8 MFMA only
+    int engine = 0;      // 0 = choose, 1 = int8 MFMA (staged), 2 = FP4 x FP8 MFMA, 3 = int8 MFMA (direct)
 };
 
 using MfmaKernelFn = void (*)(const MfmaArgs);
@@ -341,6 +570,30 @@ const MfmaTable<BITS> &mfma_table() {
 }
 
 template <int BITS>
+const MfmaTable<BITS> &mfma_direct_table() {
+    static const MfmaTable<BITS> t = [] {
+        MfmaTable<BITS> x{};
+        x.fn[0][0] = gemv_mfma_direct_kernel<BITS, 1, false, false>;
+        x.fn[0][1] = gemv_mfma_direct_kernel<BITS, 1, false, true>;
+        x.fn[0][2] = gemv_mfma_direct_kernel<BITS, 1, true, false>;
+        x.fn[1][0] = gemv_mfma_direct_kernel<BITS, 2, false, false>;
+        x.fn[1][1] = gemv_mfma_direct_kernel<BITS, 2, false, true>;
+        x.fn[1][2] = gemv_mfma_direct_kernel<BITS, 2, true, false>;
+        x.fn[2][0] = gemv_mfma_direct_kernel<BITS, 4, false, false>;
+        x.fn[2][1] = gemv_mfma_direct_kernel<BITS, 4, false, true>;
+        x.fn[2][2] = gemv_mfma_direct_kernel<BITS, 4, true, false>;
+        return x;
+    }();
+    return t;
+}
+
+template <int BITS>
+size_t mfma_direct_lds_for(int ri) {
+    return ri == 0 ? mfma_direct_lds_bytes<BITS, 1>()
+                   : (ri == 1 ? mfma_direct_lds_bytes<BITS, 2>() : mfma_direct_lds_bytes<BITS, 4>());
+}
+
+template <int BITS>
 MfmaTuning &mfma_tuning() {
     static MfmaTuning t;
     return t;
@@ -348,13 +601,14 @@ MfmaTuning &mfma_tuning() {
 
 template <int BITS>
 int mfma_init_device(int max_lds) {
-    const MfmaTable<BITS> &t = mfma_table<BITS>();
-    for (int r = 0; r < 3; ++r)
-        for (int v = 0; v < 3; ++v)
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[r][v]),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    max_lds) != hipSuccess)
-                return 2;
+    const MfmaTable<BITS> *tables[2] = {&mfma_table<BITS>(), &mfma_direct_table<BITS>()};
+    for (const MfmaTable<BITS> *t : tables)
+        for (int r = 0; r < 3; ++r)
+            for (int v = 0; v < 3; ++v)
+                if (hipFuncSetAttribute(reinterpret_cast<const void *>(t->fn[r][v]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        max_lds) != hipSuccess)
+                    return 2;
     return 0;
 }
 

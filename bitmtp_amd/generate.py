@@ -111,7 +111,6 @@ def _stats_common(prefill_time, decode_time, total_time, seq_len, out_len):
     }
 
 
-@torch.inference_mode()
 def ar_generate(atlas: GraphAtlas, input_ids: Sequence[int], max_gen_len: int = 512,
                 eos_ids: Iterable[int] = ()) -> Tuple[List[int], dict]:
     """Greedy AR decode with the width-1 graph (fast_generate.py:179-292)."""
@@ -183,7 +182,6 @@ def _exact_m1_verify(atlas: GraphAtlas, sigma: int, cache_len: int, pending: Lis
     return accept, cache_len + accept, pred
 
 
-@torch.inference_mode()
 def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: float = 0.9,
                     hybrid_m: Optional[int] = None, max_gen_len: int = 512,
                     eos_ids: Iterable[int] = (), exact_m1_verify: bool = False

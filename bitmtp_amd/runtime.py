@@ -216,6 +216,11 @@ class GraphAtlas:
                     self.get_graph(M, sigma, role)
 
     def _capture_one(self, M: int, sigma: int, role: str) -> CapturedGraph:
+        # capture keeps process-wide state tensors; they must not become inference tensors
+        with torch.inference_mode(False):
+            return self._capture_one_impl(M, sigma, role)
+
+    def _capture_one_impl(self, M: int, sigma: int, role: str) -> CapturedGraph:
         if role not in ROLES:
             raise ValueError(f"unsupported graph role: {role!r}")
         if role == "draft" and M < self.D:

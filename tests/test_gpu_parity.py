@@ -91,13 +91,14 @@ def test_launch_geometries(oracle, bits, lpr, waves, passes):
 
 
 @pytest.mark.parametrize("bits", [2, 1])
-@pytest.mark.parametrize("engine", [1, 2])
+@pytest.mark.parametrize("engine", [1, 2, 3])
 @pytest.mark.parametrize("min_width,row_tiles,k_split,passes", [
     (1, 1, 1, 1), (1, 2, 2, 0), (1, 4, 4, 0), (2, 1, 4, 0), (2, 4, 1, 3), (2, 2, 1, 2),
     (1, 1, 1, 5), (1000, 0, 0, 0),
 ])
 def test_mfma_geometries(oracle, bits, engine, min_width, row_tiles, k_split, passes):
-    """Both matrix-core kernels (1 = int8 MFMA, 2 = FP4 x FP8 MFMA): every row-tile /
+    """The matrix-core kernels (1 = int8 MFMA with staged activations, 2 = FP4 x FP8 MFMA,
+    3 = int8 MFMA with activations loaded as operands): every row-tile /
     K-split / pass combination, including a single token sent through them, and the
     dot4 kernel forced for every width (min_width 1000)."""
     from bitmtp_amd import ops as O2
