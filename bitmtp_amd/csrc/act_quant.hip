@@ -11,6 +11,7 @@
 #include <stdint.h>
 
 #include "../../include/bonsai_gemv.h"
+#include "wave_reduce.h"
 
 namespace {
 
@@ -155,11 +156,10 @@ __host__ __device__ inline int producer_threads(int nvec) {
 }
 
 // Fixed reduction order (the CPU oracle replays it): thread t accumulates its vectors
-// t, t+T, ... in turn, an xor butterfly (32,16,...,1) inside each wave, then the wave
+// t, t+T, ... in turn, an xor butterfly (1,2,...,32) inside each wave, then the wave
 // totals left to right.
 __device__ __forceinline__ double block_sum_f64(double v, double *scratch) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    v = bonsai_wave::sum64(v);  // the xor butterfly 1, 2, ..., 32 on the DPP network
     if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
     __syncthreads();
     const int waves = blockDim.x >> 6;
@@ -169,8 +169,7 @@ __device__ __forceinline__ double block_sum_f64(double v, double *scratch) {
 }
 
 __device__ __forceinline__ float block_max_f32(float v, float *scratch) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    v = bonsai_wave::max64(v);
     if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
     __syncthreads();
     const int waves = blockDim.x >> 6;

@@ -18,6 +18,7 @@
 #include <stdint.h>
 
 #include "../../include/bonsai_decode.h"
+#include "wave_reduce.h"
 
 namespace {
 
@@ -43,16 +44,8 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(x, y, c, false);
 }
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
-}
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
-}
+__device__ __forceinline__ float wave_max(float v) { return bonsai_wave::max64(v); }
+__device__ __forceinline__ float wave_sum(float v) { return bonsai_wave::sum64(v); }
 
 // ---------------------------------------------------------------------------
 // q/k RMSNorm + RoPE + KV write.  One wave per (token, head); lane i holds the
@@ -93,9 +86,7 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(RopeArgs a) {
     const bool is_q = head < a.n_heads;
     const uint16_t *w = is_q ? a.qw : a.kw;
     const float f0 = bf16_bits_to_f32(r0), f1 = bf16_bits_to_f32(r1);
-    double ss = (double)(f0 * f0) + (double)(f1 * f1);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    const double ss = bonsai_wave::sum64((double)(f0 * f0) + (double)(f1 * f1));
     const float var = (float)ss / (float)kHd;
     const float rs = 1.0f / sqrtf(var + a.eps);
     const float n0 = bf16_round(bf16_bits_to_f32(w[lane]) * bf16_round(f0 * rs));

@@ -266,7 +266,7 @@ static inline float bf16_round_f(float f) { return oracle_bf16_to_f32(oracle_f32
 
 /* Sum of fp32 squares in fp64, in the order the HIP kernel uses: T threads with
  * T = min(1024, K/8 rounded up to a multiple of 64); thread t takes the 8-element
- * vectors t, t+T, ... in turn; xor butterfly (32,16,..,1) inside each 64-thread wave;
+ * vectors t, t+T, ... in turn; xor butterfly (1,2,..,32) inside each 64-thread wave;
  * the wave totals added left to right. */
 static double sumsq_kernel_order(const float *h, int K) {
     static double lane[1024];
@@ -286,7 +286,7 @@ static double sumsq_kernel_order(const float *h, int K) {
     for (int w = 0; w < T / 64; ++w) {
         double a[64], b[64];
         for (int i = 0; i < 64; ++i) a[i] = lane[64 * w + i];
-        for (int off = 32; off > 0; off >>= 1) {
+        for (int off = 1; off < 64; off <<= 1) {
             for (int i = 0; i < 64; ++i) b[i] = a[i] + a[i ^ off];
             for (int i = 0; i < 64; ++i) a[i] = b[i];
         }
