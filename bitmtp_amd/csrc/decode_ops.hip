@@ -469,10 +469,14 @@ __global__ void draft_accept_kernel(const float *conf, int rows, float threshold
     accept[1] = rows;
 }
 
+int g_rows_per_wave = 0;  // 0 = heuristic; set through bonsai_decode_set_tuning
+
 int rows_per_wave(int M) {
-    // few rows per wave keep phase 2 short; more row groups re-read K/V from L2
-    if (M <= 4) return M;
-    if (M <= 12) return 3;
+    if (g_rows_per_wave >= 1 && g_rows_per_wave <= 4) return g_rows_per_wave < M ? g_rows_per_wave : (M < 4 ? M : 4);
+    // few rows per wave keep the waves short; more row groups re-read K/V from L2 (measured:
+    // two rows per wave up to a dozen rows, four above)
+    if (M <= 2) return M;
+    if (M <= 12) return 2;
     return 4;
 }
 
@@ -511,6 +515,10 @@ extern "C" int bonsai_qk_norm_rope_kv_write(const void *xqkv, const void *q_norm
     hipLaunchKernelGGL(qk_norm_rope_kernel, dim3((total_heads + 3) / 4, M), dim3(256), 0,
                        static_cast<hipStream_t>(stream), a);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" void bonsai_decode_set_tuning(int rows_per_wave_override) {
+    g_rows_per_wave = rows_per_wave_override;
 }
 
 extern "C" int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int slots) {

@@ -62,6 +62,10 @@ int bonsai_qk_norm_rope_kv_write(const void *xqkv, const void *q_norm_w, const v
                                  void *v_layer, int M, int n_heads, int n_kv, int slots,
                                  int write_slot, int max_pos, void *stream);
 
+/* Process-wide tuning of the attention launch geometry: query rows per wave (1..4), 0 =
+ * built-in heuristic.  No counterpart in the reference; results do not depend on it. */
+void bonsai_decode_set_tuning(int rows_per_wave);
+
 /* Bytes of scratch `bonsai_decode_attention` needs for the given shape. */
 int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int slots);
 
