@@ -341,3 +341,47 @@ def test_eos_stops_generation(tiny):
     hy, _ = generate.hybrid_generate(atlas, prompt, max_gen_len=24, eos_ids=[eos],
                                      exact_m1_verify=True)
     assert hy == ar[:first]
+
+
+def test_segment_migration_keeps_the_sequence(tiny):
+    """Moving the live history to a larger segment's buffer (fast_runtime.py:510-521) and
+    decoding on from there gives the same tokens as staying put."""
+    from bitmtp_amd import generate
+    model, atlas = tiny
+    prompt = list(range(11, 45))
+    ar, _ = generate.ar_generate(atlas, prompt, max_gen_len=12)       # lives in segment 64
+    assert atlas.select_segment(len(prompt) + 12 + atlas.M_max) == 64
+    # replay the same decode by hand, migrating 64 -> 256 after four tokens
+    sigma = 64
+    tok = generate.prefill(atlas, prompt, sigma)
+    cache_len = len(prompt)
+    out = [tok]
+    for step in range(11):
+        if step == 4:
+            atlas.migrate_segment(sigma, 256, cache_len)
+            sigma = 256
+        g = atlas.get_graph(1, sigma, "ar")
+        atlas.replay(g, [tok], [cache_len], cache_len)
+        atlas.commit_kv(sigma, cache_len, 1)
+        cache_len += 1
+        toks, _, _ = atlas.read_outputs(g)
+        tok = int(toks[0])
+        out.append(tok)
+    assert out == ar
+
+
+def test_replay_argument_checks(tiny):
+    model, atlas = tiny
+    g = atlas.get_graph(9, 64, "verify")
+    with pytest.raises(ValueError):
+        atlas.replay(g, [1, 2, 3], [0, 1, 2], 5)
+    with pytest.raises(RuntimeError, match="committed anchor"):
+        atlas.replay(g, [1] * 9, list(range(9)), 0)
+    with pytest.raises(RuntimeError):
+        atlas.replay(g, [1] * 9, list(range(9)), 65)
+    with pytest.raises(RuntimeError):
+        atlas.commit_kv(64, 60, 9)
+    with pytest.raises(ValueError):
+        atlas.get_graph(4, 64, "draft")
+    with pytest.raises(KeyError):
+        atlas.kv(100)
