@@ -34,6 +34,8 @@ HIPCC_FLAGS = [
     # MFMA results go to ordinary VGPRs: the scale-accumulate epilogue consumes them
     # at once and v_accvgpr_read copies would cost four VALU slots per tile
     "-mllvm", "--amdgpu-mfma-vgpr-form",
+    # scalar kernel arguments arrive in SGPRs with the wave instead of through a load
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 
