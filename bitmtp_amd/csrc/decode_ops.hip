@@ -67,7 +67,14 @@ struct RopeArgs {
     int M, n_heads, n_kv, slots, write_slot, max_pos;
 };
 
-__global__ void __launch_bounds__(256) qk_norm_rope_kernel(RopeArgs a) {
+__global__ void __launch_bounds__(256)
+qk_norm_rope_kernel(const uint16_t *pxqkv, const uint16_t *pqw, const uint16_t *pkw,
+                    const uint16_t *pcos, const uint16_t *psin, const int32_t *ppos,
+                    uint16_t *pq, uint16_t *pk, uint16_t *pv, float peps, int pM, int pheads,
+                    int pkv, int pslots, int pwrite, int pmaxpos) {
+    // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
+    const RopeArgs a{pxqkv, pqw, pkw, pcos, psin, ppos, pq, pk, pv, peps,
+                     pM, pheads, pkv, pslots, pwrite, pmaxpos};
     const int lane = threadIdx.x & 63;
     const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int m = blockIdx.y;
@@ -132,7 +139,13 @@ struct AttnArgs {
 };
 
 template <int RW>
-__global__ void __launch_bounds__(64) attn_partial_kernel(AttnArgs a) {
+__global__ void __launch_bounds__(64)
+attn_partial_kernel(const uint32_t *pq, const uint32_t *pk, const uint32_t *pv, const int32_t *pmeta,
+                    float *ppart, float pscale, int pM, int pheads, int pkv, int phpg, int pslots,
+                    int psigma, int pchunks, int prow_groups) {
+    // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
+    const AttnArgs a{pq, pk, pv, pmeta, ppart, pscale, pM, pheads, pkv, phpg, pslots,
+                     psigma, pchunks, prow_groups};
     __shared__ __attribute__((aligned(16))) float p_lds[RW][kChunk];
     const int lane = threadIdx.x;
     int id = blockIdx.x;
@@ -254,7 +267,10 @@ constexpr int kCombineMaxVec = 2;      // 8-element vectors per thread: up to 32
 constexpr int kCombineMaxHeads = kCombineThreads * kCombineMaxVec / (kHd / 8);
 constexpr int kCombineMaxChunks = 136;  // sigma + M up to 8704 slots
 
-__global__ void __launch_bounds__(kCombineThreads) attn_combine_kernel(CombineArgs a) {
+__global__ void __launch_bounds__(kCombineThreads)
+attn_combine_kernel(const float *ppart, const int32_t *pmeta, uint16_t *pout, int8_t *pq, float *ps,
+                    int pM, int pheads, int pchunks, int psigma) {
+    const CombineArgs a{ppart, pmeta, pout, pq, ps, pM, pheads, pchunks, psigma};
     __shared__ float wgt[kCombineMaxHeads * kCombineMaxChunks];  // becomes the chunk weights
     __shared__ float lsum[kCombineMaxHeads * kCombineMaxChunks];
     __shared__ float max_scratch[kCombineThreads / 64];
@@ -513,7 +529,9 @@ extern "C" int bonsai_qk_norm_rope_kv_write(const void *xqkv, const void *q_norm
     a.max_pos = max_pos;
     const int total_heads = n_heads + 2 * n_kv;
     hipLaunchKernelGGL(qk_norm_rope_kernel, dim3((total_heads + 3) / 4, M), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), a);
+                       static_cast<hipStream_t>(stream), a.xqkv, a.qw, a.kw, a.cos_t, a.sin_t,
+                       a.positions, a.q_out, a.k_layer, a.v_layer, a.eps, a.M, a.n_heads, a.n_kv,
+                       a.slots, a.write_slot, a.max_pos);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 
@@ -558,12 +576,17 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
     a.row_groups = (M + rw - 1) / rw;
     const AttnArgs &launch = a;
     const int blocks = n_kv * a.n_chunks * a.hpg * a.row_groups;
+#define ATTN_ARGS                                                                             \
+    launch.q, launch.k_layer, launch.v_layer, launch.meta, launch.part, launch.scale_log2e,      \
+        launch.M, launch.n_heads, launch.n_kv, launch.hpg, launch.slots, launch.sigma,           \
+        launch.n_chunks, launch.row_groups
     switch (rw) {
-        case 1: hipLaunchKernelGGL(attn_partial_kernel<1>, dim3(blocks), dim3(64), 0, st, launch); break;
-        case 2: hipLaunchKernelGGL(attn_partial_kernel<2>, dim3(blocks), dim3(64), 0, st, launch); break;
-        case 3: hipLaunchKernelGGL(attn_partial_kernel<3>, dim3(blocks), dim3(64), 0, st, launch); break;
-        default: hipLaunchKernelGGL(attn_partial_kernel<4>, dim3(blocks), dim3(64), 0, st, launch); break;
+        case 1: hipLaunchKernelGGL(attn_partial_kernel<1>, dim3(blocks), dim3(64), 0, st, ATTN_ARGS); break;
+        case 2: hipLaunchKernelGGL(attn_partial_kernel<2>, dim3(blocks), dim3(64), 0, st, ATTN_ARGS); break;
+        case 3: hipLaunchKernelGGL(attn_partial_kernel<3>, dim3(blocks), dim3(64), 0, st, ATTN_ARGS); break;
+        default: hipLaunchKernelGGL(attn_partial_kernel<4>, dim3(blocks), dim3(64), 0, st, ATTN_ARGS); break;
     }
+#undef ATTN_ARGS
     if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
     CombineArgs c;
     c.part = launch.part;
@@ -575,7 +598,8 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
     c.n_heads = n_heads;
     c.n_chunks = a.n_chunks;
     c.sigma = sigma;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(M), dim3(kCombineThreads), 0, st, c);
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(M), dim3(kCombineThreads), 0, st, c.part, c.meta,
+                       c.out_bf16, c.out_q, c.out_s, c.M, c.n_heads, c.n_chunks, c.sigma);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 

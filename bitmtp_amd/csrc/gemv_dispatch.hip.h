@@ -117,7 +117,8 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
                                 : (direct ? mfma_direct_table<BITS>().fn[ri][variant]
                                           : mfma_table<BITS>().fn[ri][variant]);
     hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(kMfmaThreads, 1, 1), lds_for(ri, mt),
-                       stream, args);
+                       stream, args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
+                       args.mt, args.ks_log2, args.out_f32, args.passes, args.div_magic);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

@@ -58,7 +58,11 @@ __device__ __forceinline__ void int8x4_to_fp8_planes(uint32_t x, uint32_t &hi, u
 }
 
 template <int BITS, int R, bool G32, bool SF16>
-__global__ void __launch_bounds__(kMfmaThreads) gemv_fp4_kernel(const MfmaArgs a) {
+__global__ void __launch_bounds__(kMfmaThreads) gemv_fp4_kernel
+(const int8_t *pA, const uint8_t *pB, void *pout, const float *ps, const uint16_t *pws, int pM,
+ int pN, int pK, int pmt, int pks_log2, int pout_f32, int ppasses, uint32_t pdiv_magic) {
+    // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
+    const MfmaArgs a{pA, pB, pout, ps, pws, pM, pN, pK, pmt, pks_log2, pout_f32, ppasses, pdiv_magic};
     using MF = MfmaFmt<BITS>;
     extern __shared__ __align__(16) unsigned char smem[];
 

@@ -70,7 +70,11 @@ __host__ __device__ inline size_t mfma_lds_bytes(int mt, int K) {
 }
 
 template <int BITS, int R, bool G32, bool SF16>
-__global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel(const MfmaArgs a) {
+__global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel
+(const int8_t *pA, const uint8_t *pB, void *pout, const float *ps, const uint16_t *pws, int pM,
+ int pN, int pK, int pmt, int pks_log2, int pout_f32, int ppasses, uint32_t pdiv_magic) {
+    // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
+    const MfmaArgs a{pA, pB, pout, ps, pws, pM, pN, pK, pmt, pks_log2, pout_f32, ppasses, pdiv_magic};
     using MF = MfmaFmt<BITS>;
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -318,7 +322,11 @@ __host__ __device__ inline size_t mfma_direct_lds_bytes() {
 }
 
 template <int BITS, int R, bool G32, bool SF16>
-__global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_direct_kernel(const MfmaArgs a) {
+__global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_direct_kernel
+(const int8_t *pA, const uint8_t *pB, void *pout, const float *ps, const uint16_t *pws, int pM,
+ int pN, int pK, int pmt, int pks_log2, int pout_f32, int ppasses, uint32_t pdiv_magic) {
+    // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
+    const MfmaArgs a{pA, pB, pout, ps, pws, pM, pN, pK, pmt, pks_log2, pout_f32, ppasses, pdiv_magic};
     using MF = MfmaFmt<BITS>;
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -543,7 +551,8 @@ struct MfmaTuning {
     int engine = 0;      // 0 = choose, 1 = int8 MFMA (staged), 2 = FP4 x FP8 MFMA, 3 = int8 MFMA (direct)
 };
 
-using MfmaKernelFn = void (*)(const MfmaArgs);
+using MfmaKernelFn = void (*)(const int8_t *, const uint8_t *, void *, const float *,
+                              const uint16_t *, int, int, int, int, int, int, int, uint32_t);
 
 template <int BITS>
 struct MfmaTable {
