@@ -158,21 +158,19 @@ __host__ __device__ inline int producer_threads(int nvec) {
 // Fixed reduction order (the CPU oracle replays it): thread t accumulates its vectors
 // t, t+T, ... in turn, an xor butterfly (1,2,...,32) inside each wave, then the wave
 // totals left to right.
-__device__ __forceinline__ double block_sum_f64(double v, double *scratch) {
+__device__ __forceinline__ double block_sum_f64(double v, double *scratch, int waves) {
     v = bonsai_wave::sum64(v);  // the xor butterfly 1, 2, ..., 32 on the DPP network
     if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
     __syncthreads();
-    const int waves = blockDim.x >> 6;
     double t = scratch[0];
     for (int w = 1; w < waves; ++w) t += scratch[w];
     return t;
 }
 
-__device__ __forceinline__ float block_max_f32(float v, float *scratch) {
+__device__ __forceinline__ float block_max_f32(float v, float *scratch, int waves) {
     v = bonsai_wave::max64(v);
     if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
     __syncthreads();
-    const int waves = blockDim.x >> 6;
     float t = scratch[0];
     for (int w = 1; w < waves; ++w) t = fmaxf(t, scratch[w]);
     return t;
@@ -199,12 +197,12 @@ __device__ __forceinline__ void unpack8_bf16(const uint4 raw, float out[8]) {
 template <bool ADD, int VPT>
 __global__ void __launch_bounds__(kMaxProducerThreads)
 rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t *w, float eps,
-                     uint16_t *h_out, int8_t *q, float *s, int K) {
+                     uint16_t *h_out, int8_t *q, float *s, int K, int T) {
+    // T = workgroup size, passed explicitly: reading blockDim costs a load at kernel start
     __shared__ double sum_scratch[kMaxProducerWaves];
     __shared__ float max_scratch[kMaxProducerWaves];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
-    const int T = blockDim.x;
     const int nvec = K / 8;
     const uint4 *xrow = reinterpret_cast<const uint4 *>(x + (size_t)m * K);
     const uint4 *rrow = ADD ? reinterpret_cast<const uint4 *>(residual + (size_t)m * K) : nullptr;
@@ -248,7 +246,7 @@ rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t
             }
         }
     }
-    const double total = block_sum_f64(ss, sum_scratch);
+    const double total = block_sum_f64(ss, sum_scratch, T >> 6);
     const float var = (float)total / (float)K;
     const float rs = 1.0f / sqrtf(var + eps);
 
@@ -264,7 +262,7 @@ rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t
             if (v < nvec) amax = fmaxf(amax, fabsf(h[i][e]));
         }
     }
-    amax = block_max_f32(amax, max_scratch);
+    amax = block_max_f32(amax, max_scratch, T >> 6);
     const float recip = 1.0f / fmaxf(amax, 1e-5f);
     const float sval = recip * 127.0f;
     if (tid == 0) s[m] = sval;
@@ -279,11 +277,10 @@ rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t
 // inner = bf16( fp32(bf16(silu(gate))) * up ), gate = gu[m][0..F), up = gu[m][F..2F)
 template <int VPT>
 __global__ void __launch_bounds__(kMaxProducerThreads)
-silu_mul_quant_kernel(const uint16_t *gu, int8_t *q, float *s, int F) {
+silu_mul_quant_kernel(const uint16_t *gu, int8_t *q, float *s, int F, int T) {
     __shared__ float max_scratch[kMaxProducerWaves];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
-    const int T = blockDim.x;
     const int nvec = F / 8;
     const uint4 *grow = reinterpret_cast<const uint4 *>(gu + (size_t)m * 2 * F);
     const uint4 *urow = reinterpret_cast<const uint4 *>(gu + (size_t)m * 2 * F + F);
@@ -310,7 +307,7 @@ silu_mul_quant_kernel(const uint16_t *gu, int8_t *q, float *s, int F) {
             if (v < nvec) amax = fmaxf(amax, fabsf(nf[i][e]));
         }
     }
-    amax = block_max_f32(amax, max_scratch);
+    amax = block_max_f32(amax, max_scratch, T >> 6);
     const float recip = 1.0f / fmaxf(amax, 1e-5f);
     const float sval = recip * 127.0f;
     if (tid == 0) s[m] = sval;
@@ -339,10 +336,10 @@ void launch_rmsnorm(const uint16_t *x, const uint16_t *r, const uint16_t *w, flo
     const int nvec = K / 8;
     const dim3 grid(M), block(producer_threads(nvec));
     switch (producer_vpt(nvec)) {
-        case 1: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 1>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
-        case 2: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 2>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
-        case 4: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 4>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
-        default: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 8>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K); break;
+        case 1: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 1>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
+        case 2: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 2>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
+        case 4: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 4>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
+        default: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 8>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
     }
 }
 
@@ -403,10 +400,10 @@ extern "C" int bonsai_silu_mul_quant_int8(const void *gate_up, int8_t *q, float 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint16_t *gu = reinterpret_cast<const uint16_t *>(gate_up);
     switch (producer_vpt(nvec)) {
-        case 1: hipLaunchKernelGGL(silu_mul_quant_kernel<1>, grid, block, 0, st, gu, q, s, F); break;
-        case 2: hipLaunchKernelGGL(silu_mul_quant_kernel<2>, grid, block, 0, st, gu, q, s, F); break;
-        case 4: hipLaunchKernelGGL(silu_mul_quant_kernel<4>, grid, block, 0, st, gu, q, s, F); break;
-        default: hipLaunchKernelGGL(silu_mul_quant_kernel<8>, grid, block, 0, st, gu, q, s, F); break;
+        case 1: hipLaunchKernelGGL(silu_mul_quant_kernel<1>, grid, block, 0, st, gu, q, s, F, (int)block.x); break;
+        case 2: hipLaunchKernelGGL(silu_mul_quant_kernel<2>, grid, block, 0, st, gu, q, s, F, (int)block.x); break;
+        case 4: hipLaunchKernelGGL(silu_mul_quant_kernel<4>, grid, block, 0, st, gu, q, s, F, (int)block.x); break;
+        default: hipLaunchKernelGGL(silu_mul_quant_kernel<8>, grid, block, 0, st, gu, q, s, F, (int)block.x); break;
     }
     return hipGetLastError() == hipSuccess ? BONSAI_OK : BONSAI_ERR_LAUNCH;
 }

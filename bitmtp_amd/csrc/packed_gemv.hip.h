@@ -103,7 +103,7 @@ template <int BITS, int MT, int U, bool G32, bool SF16>
 __global__ void __launch_bounds__(kMaxThreads)
 gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *ps,
                  const uint16_t *pws, int pM, int pN, int pK, int plpr_log2, int ppasses,
-                 int pout_f32, uint32_t pdiv_magic) {
+                 int pout_f32, uint32_t pdiv_magic, int pthreads) {
     // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
     const GemvArgs a{pA, pB, pout, ps, pws, pM, pN, pK, plpr_log2, ppasses, pout_f32, pdiv_magic};
     using F = Fmt<BITS>;
@@ -117,7 +117,7 @@ gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *p
     int *asum = reinterpret_cast<int *>(smem);
 
     const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
+    const int nthreads = pthreads;  // the workgroup size, as a parameter: blockDim is a load
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int nwaves = nthreads >> 6;
@@ -295,7 +295,7 @@ struct Tuning {
 };
 
 using KernelFn = void (*)(const int8_t *, const uint8_t *, void *, const float *, const uint16_t *,
-                          int, int, int, int, int, int, uint32_t);
+                          int, int, int, int, int, int, uint32_t, int);
 constexpr int kBatchKinds = 3;  // U = 1, 2, 4
 constexpr int kVariants = 3;    // 0: bf16 scales, 1: fp16 scales, 2: int32 group sums
 
@@ -481,7 +481,7 @@ int launch_gemv_dot4(const int8_t *A, const uint8_t *B, void *out, const float *
     const KernelFn fn = kernel_table<BITS>().fn[g.mt - 1][g.batch_index][variant];
     hipLaunchKernelGGL(fn, dim3(g.grid_x, g.ntiles, 1), dim3(g.waves * 64, 1, 1), g.lds, stream,
                        args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
-                       args.lpr_log2, args.passes, args.out_f32, args.div_magic);
+                       args.lpr_log2, args.passes, args.out_f32, args.div_magic, g.waves * 64);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
