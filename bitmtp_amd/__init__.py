@@ -6,7 +6,7 @@ from .ops import (  # noqa: F401
     init_kernels, load_actq_kernel, load_q1_kernel, load_t2_kernel,
     packed_gemv_ex, packed_int8_linear, q1g128_int8xint1_linear, q1g128_w1a16_linear,
     quant_input, t2g128_int8xint2_linear,
-    fused_add_norm_quant, fused_norm_quant, silu_mul_quant,
+    add_rmsnorm, fused_add_norm_quant, fused_norm_quant, silu_mul_quant,
 )
 from .packing import (  # noqa: F401
     merge_packed_rows, pack_q1_g128, pack_t2_g128, unpack_q1_g128, unpack_t2_g128,
@@ -17,5 +17,5 @@ __all__ = [
     "packed_gemv_ex", "packed_int8_linear", "q1g128_int8xint1_linear", "q1g128_w1a16_linear",
     "quant_input", "t2g128_int8xint2_linear", "pack_q1_g128", "pack_t2_g128",
     "unpack_q1_g128", "unpack_t2_g128", "OUT_BF16", "OUT_F32", "OUT_G32",
-    "fused_add_norm_quant", "fused_norm_quant", "silu_mul_quant", "merge_packed_rows",
+    "add_rmsnorm", "fused_add_norm_quant", "fused_norm_quant", "silu_mul_quant", "merge_packed_rows",
 ]

@@ -363,14 +363,16 @@ def expected_packed_keys(args) -> Dict[str, Tuple[torch.dtype, Tuple[int, ...]]]
 
 
 def load_packed_state(ckpt_dir: str) -> Tuple[object, Dict[str, torch.Tensor]]:
-    """Read and validate ``model_state_t2g128.pt`` (CPU tensors).  Missing or unexpected keys
+    """Read and validate ``model_state_t2g128.pt`` (``model_state_q1g128.pt`` for a sign-weight
+    checkpoint; CPU tensors).  Missing or unexpected keys
     and wrong dtypes / shapes raise, like ``build_model`` (generate.py:49-68)."""
     args = load_args_from_ckpt(ckpt_dir, use_kernel=True)
-    if args.kernel_kind != "t2g128":
-        raise ValueError("the MI355X decoder loads ternary (t2g128) checkpoints")
-    if not args.tie_word_embeddings:
+    if args.kernel_kind not in ("t2g128", "q1"):
+        raise ValueError(f"unknown kernel_kind {args.kernel_kind!r} in bonsai_gpu_config.json")
+    if args.kernel_kind == "t2g128" and not args.tie_word_embeddings:
         raise ValueError("the packed T2 head is the tied embedding; untied checkpoints are not supported")
-    path = os.path.join(ckpt_dir, "model_state_t2g128.pt")
+    path = os.path.join(ckpt_dir, "model_state_t2g128.pt" if args.kernel_kind == "t2g128"
+                        else "model_state_q1g128.pt")
     sd = torch.load(path, map_location="cpu", weights_only=True)
     want = expected_packed_keys(args)
     missing = [k for k in want if k not in sd]
@@ -387,17 +389,21 @@ def load_packed_state(ckpt_dir: str) -> Tuple[object, Dict[str, torch.Tensor]]:
 
 def load_decoder(ckpt_dir: str, device="cuda"):
     """Packed checkpoint -> ``BonsaiDecoder`` with q|k|v and gate|up merged along the output
-    rows (``prepare_merged_weights``, model.py:931-956,1042-1051) and the tied head packed on
-    its ternary grid, padded to whole 128-row tiles (``prepare_t2_lm_head``, model.py:1222-1243)."""
-    from .model import BonsaiDecoder, LayerWeights, PackedLinear, head_rows_for
+    rows (``prepare_merged_weights``, model.py:931-956,1042-1051).  A ternary checkpoint gets
+    the tied head packed on its ternary grid, padded to whole 128-row tiles
+    (``prepare_t2_lm_head``, model.py:1222-1243); a sign-weight ("q1") checkpoint keeps the
+    output projection in bf16 (the tied embedding, or ``lm_head.weight`` when untied), as the
+    reference's graphs do (fast_runtime.py:175-178)."""
+    from .model import BonsaiDecoder, LayerWeights, PackedLinear, head_rows_for, kind_bits
     args, sd = load_packed_state(ckpt_dir)
     dev = torch.device(device)
+    bits = kind_bits(args.kernel_kind)
 
     def lin(prefix: str) -> Tuple[torch.Tensor, torch.Tensor]:
         return sd[prefix + ".weight"], sd[prefix + ".weight_scale"]
 
     def to_dev(pair) -> PackedLinear:
-        return PackedLinear(pair[0].contiguous().to(dev), pair[1].contiguous().to(dev))
+        return PackedLinear(pair[0].contiguous().to(dev), pair[1].contiguous().to(dev), bits)
 
     layers = []
     for i in range(args.n_layers):
@@ -411,6 +417,13 @@ def load_decoder(ckpt_dir: str, device="cuda"):
             post_attention_layernorm=sd[f"layers.{i}.post_attention_layernorm.weight"].to(dev),
             q_norm=sd[a + "q_norm.weight"].to(dev), k_norm=sd[a + "k_norm.weight"].to(dev)))
     embed = sd["embed_tokens.weight"].to(dev).contiguous()
+    if bits == 1:
+        head_bf16 = None
+        if not args.tie_word_embeddings:
+            if "lm_head.weight" not in sd:
+                raise RuntimeError("Missing weights: ['lm_head.weight']")
+            head_bf16 = sd["lm_head.weight"].to(dev).contiguous()
+        return BonsaiDecoder(args, layers, embed, sd["norm.weight"].to(dev), None, head_bf16)
     rows = head_rows_for(args.vocab_size)
     padded = torch.zeros(rows, args.dim, dtype=torch.bfloat16, device=dev)
     padded[: args.vocab_size].copy_(embed)

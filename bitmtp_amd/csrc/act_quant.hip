@@ -197,7 +197,8 @@ __device__ __forceinline__ void unpack8_bf16(const uint4 raw, float out[8]) {
 template <bool ADD, int VPT>
 __global__ void __launch_bounds__(kMaxProducerThreads)
 rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t *w, float eps,
-                     uint16_t *h_out, int8_t *q, float *s, int K, int T) {
+                     uint16_t *h_out, uint16_t *n_out, int8_t *q, float *s, int K, int T) {
+    // n_out (optional): the normalised row in bf16; q / s (optional): its quantisation.
     // T = workgroup size, passed explicitly: reading blockDim costs a load at kernel start
     __shared__ double sum_scratch[kMaxProducerWaves];
     __shared__ float max_scratch[kMaxProducerWaves];
@@ -229,7 +230,7 @@ rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t
             unpack8_bf16(rr[i], r);
 #pragma unroll
             for (int e = 0; e < 8; ++e) h[i][e] = bf16_round(h[i][e] + r[e]);
-            if (v < nvec) {
+            if (v < nvec && h_out != nullptr) {
                 uint4 o;
                 o.x = f32_to_bf16_bits(h[i][0]) | (f32_to_bf16_bits(h[i][1]) << 16);
                 o.y = f32_to_bf16_bits(h[i][2]) | (f32_to_bf16_bits(h[i][3]) << 16);
@@ -261,7 +262,16 @@ rmsnorm_quant_kernel(const uint16_t *x, const uint16_t *residual, const uint16_t
             h[i][e] = bf16_round(wv[e] * bf16_round(h[i][e] * rs));
             if (v < nvec) amax = fmaxf(amax, fabsf(h[i][e]));
         }
+        if (n_out != nullptr && v < nvec) {
+            uint4 o;
+            o.x = f32_to_bf16_bits(h[i][0]) | (f32_to_bf16_bits(h[i][1]) << 16);
+            o.y = f32_to_bf16_bits(h[i][2]) | (f32_to_bf16_bits(h[i][3]) << 16);
+            o.z = f32_to_bf16_bits(h[i][4]) | (f32_to_bf16_bits(h[i][5]) << 16);
+            o.w = f32_to_bf16_bits(h[i][6]) | (f32_to_bf16_bits(h[i][7]) << 16);
+            reinterpret_cast<uint4 *>(n_out + (size_t)m * K)[v] = o;
+        }
     }
+    if (q == nullptr) return;  // norm only (uniform over the grid)
     amax = block_max_f32(amax, max_scratch, T >> 6);
     const float recip = 1.0f / fmaxf(amax, 1e-5f);
     const float sval = recip * 127.0f;
@@ -332,14 +342,15 @@ constexpr int kMaxProducerK = 8 * kMaxProducerThreads * 8;  // VPT <= 8
 
 template <bool ADD>
 void launch_rmsnorm(const uint16_t *x, const uint16_t *r, const uint16_t *w, float eps,
-                    uint16_t *h_out, int8_t *q, float *s, int M, int K, hipStream_t st) {
+                    uint16_t *h_out, uint16_t *n_out, int8_t *q, float *s, int M, int K,
+                    hipStream_t st) {
     const int nvec = K / 8;
     const dim3 grid(M), block(producer_threads(nvec));
     switch (producer_vpt(nvec)) {
-        case 1: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 1>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
-        case 2: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 2>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
-        case 4: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 4>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
-        default: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 8>), grid, block, 0, st, x, r, w, eps, h_out, q, s, K, (int)block.x); break;
+        case 1: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 1>), grid, block, 0, st, x, r, w, eps, h_out, n_out, q, s, K, (int)block.x); break;
+        case 2: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 2>), grid, block, 0, st, x, r, w, eps, h_out, n_out, q, s, K, (int)block.x); break;
+        case 4: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 4>), grid, block, 0, st, x, r, w, eps, h_out, n_out, q, s, K, (int)block.x); break;
+        default: hipLaunchKernelGGL((rmsnorm_quant_kernel<ADD, 8>), grid, block, 0, st, x, r, w, eps, h_out, n_out, q, s, K, (int)block.x); break;
     }
 }
 
@@ -371,7 +382,7 @@ extern "C" int bonsai_rmsnorm_quant_int8(const void *x, const void *w, float eps
     if (x == nullptr || w == nullptr || q == nullptr || s == nullptr) return BONSAI_ERR_ARG;
     if (M < 1 || K < 8 || K % 8 != 0 || K > kMaxProducerK) return BONSAI_ERR_ARG;
     launch_rmsnorm<false>(reinterpret_cast<const uint16_t *>(x), nullptr,
-                          reinterpret_cast<const uint16_t *>(w), eps, nullptr, q, s, M, K,
+                          reinterpret_cast<const uint16_t *>(w), eps, nullptr, nullptr, q, s, M, K,
                           static_cast<hipStream_t>(stream));
     return hipGetLastError() == hipSuccess ? BONSAI_OK : BONSAI_ERR_LAUNCH;
 }
@@ -386,8 +397,26 @@ extern "C" int bonsai_add_rmsnorm_quant_int8(const void *x, const void *residual
     launch_rmsnorm<true>(reinterpret_cast<const uint16_t *>(x),
                          reinterpret_cast<const uint16_t *>(residual),
                          reinterpret_cast<const uint16_t *>(w), eps,
-                         reinterpret_cast<uint16_t *>(h_out), q, s, M, K,
+                         reinterpret_cast<uint16_t *>(h_out), nullptr, q, s, M, K,
                          static_cast<hipStream_t>(stream));
+    return hipGetLastError() == hipSuccess ? BONSAI_OK : BONSAI_ERR_LAUNCH;
+}
+
+extern "C" int bonsai_add_rmsnorm_bf16(const void *x, const void *residual, const void *w, float eps,
+                                       void *h_out, void *n_out, int M, int K, void *stream) {
+    if (x == nullptr || w == nullptr || n_out == nullptr) return BONSAI_ERR_ARG;
+    if (M < 1 || K < 8 || K % 8 != 0 || K > kMaxProducerK) return BONSAI_ERR_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (residual != nullptr)
+        launch_rmsnorm<true>(reinterpret_cast<const uint16_t *>(x),
+                             reinterpret_cast<const uint16_t *>(residual),
+                             reinterpret_cast<const uint16_t *>(w), eps,
+                             reinterpret_cast<uint16_t *>(h_out),
+                             reinterpret_cast<uint16_t *>(n_out), nullptr, nullptr, M, K, st);
+    else
+        launch_rmsnorm<false>(reinterpret_cast<const uint16_t *>(x), nullptr,
+                              reinterpret_cast<const uint16_t *>(w), eps, nullptr,
+                              reinterpret_cast<uint16_t *>(n_out), nullptr, nullptr, M, K, st);
     return hipGetLastError() == hipSuccess ? BONSAI_OK : BONSAI_ERR_LAUNCH;
 }
 

@@ -8,6 +8,7 @@
 //   kv_commit_kernel      workspace rows -> history rows (fast_runtime.py:467-508)
 //   draft_rows_kernel / draft_accept_kernel   argmax + confidence chain
 //                         (src/bonsai_sft/gpu/fast_generate.py:111-130)
+//   bf16_linear_kernel    bf16 lm_head of a sign-weight backbone (model.py:1296)
 //
 // Attention is HBM/L2-bound integer-free fp work: per layer it reads
 // 2 * n_kv * (cache_len + M) * 256 bytes of KV once per query-head group.  The mask
@@ -485,6 +486,110 @@ __global__ void draft_accept_kernel(const float *conf, int rows, float threshold
     accept[1] = rows;
 }
 
+// ---------------------------------------------------------------------------
+// bf16 output projection: out[m][n] = sum_k x[m][k] * w[n][k], the lm_head of a sign-weight
+// backbone (`_lm_head`, precision "bf16": F.linear(h, W), src/bonsai_sft/gpu/model.py:1296).
+// HBM-bound on w (2 N K bytes, read once).  The M <= 16 token rows sit in LDS; the waves of
+// a workgroup split K, each streams its slice of 16 weight rows straight into the B operand
+// of v_mfma_f32_16x16x32_bf16 (lane = (row, k-block): 32 contiguous bytes per pair of
+// MFMAs, so the four lanes of a row cover one 128-byte line) and the workgroup adds the
+// slices' partial tiles in wave order.  Workgroups stride over the 16-row tiles.
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kLinMaxWaves = 8;
+constexpr int kLinTokens = 16;
+constexpr int kLinUnroll = 4;  // pairs of 16-byte loads in flight per lane
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 v) {
+    bf16x8_t r;
+    __builtin_memcpy(&r, &v, 16);
+    return r;
+}
+
+__host__ __device__ inline size_t lin_lds_bytes(int M, int K, int nwaves) {
+    return (size_t)M * (2 * K + 16) + (size_t)2 * nwaves * 256 * sizeof(float);
+}
+
+__global__ void __launch_bounds__(kLinMaxWaves * 64)
+bf16_linear_kernel(const uint16_t *x, const uint16_t *w, uint16_t *out, int M, int N, int K,
+                   int nwaves, int ntiles, int grid) {
+    extern __shared__ __align__(16) unsigned char lin_smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pitch = 2 * K + 16;  // +16 bytes: consecutive tokens start four banks apart
+    float *part = reinterpret_cast<float *>(lin_smem + (size_t)M * pitch);  // [2][nwaves][4][64]
+
+    const int vec_per_row = K / 8;
+    for (int v = tid; v < M * vec_per_row; v += nwaves * 64) {
+        const int m = v / vec_per_row, c = v - m * vec_per_row;
+        *reinterpret_cast<uint4 *>(lin_smem + (size_t)m * pitch + (size_t)c * 16) =
+            reinterpret_cast<const uint4 *>(x + (size_t)m * K)[c];
+    }
+    __syncthreads();
+
+    const int row_l = lane & 15, kb = lane >> 4;
+    const int ksl = K / nwaves;    // elements of K per wave, a multiple of 64
+    const int npairs = ksl / 64;
+    const int k_base = wave * ksl + 16 * kb;
+    // operand rows past M alias the last token; their products are never stored
+    const int tok = row_l < M ? row_l : M - 1;
+    const unsigned char *xl = lin_smem + (size_t)tok * pitch + (size_t)k_base * 2;
+    int buf = 0;
+    for (int tile = blockIdx.x; tile < ntiles; tile += grid) {
+        int row = tile * 16 + row_l;
+        row = row < N ? row : N - 1;
+        const uint4 *wl = reinterpret_cast<const uint4 *>(w + (size_t)row * K + k_base);
+        f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int p0 = 0; p0 < npairs; p0 += kLinUnroll) {
+            uint4 wr[kLinUnroll][2];
+#pragma unroll
+            for (int u = 0; u < kLinUnroll; ++u)
+                if (p0 + u < npairs) {
+                    wr[u][0] = wl[(p0 + u) * 8];
+                    wr[u][1] = wl[(p0 + u) * 8 + 1];
+                }
+#pragma unroll
+            for (int u = 0; u < kLinUnroll; ++u)
+                if (p0 + u < npairs) {
+                    const uint4 x0 = *reinterpret_cast<const uint4 *>(xl + (size_t)(p0 + u) * 128);
+                    const uint4 x1 = *reinterpret_cast<const uint4 *>(xl + (size_t)(p0 + u) * 128 + 16);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x0), as_bf16x8(wr[u][0]),
+                                                                  acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x1), as_bf16x8(wr[u][1]),
+                                                                  acc, 0, 0, 0);
+                }
+        }
+        // acc[r]: token 4*kb + r, weight row row_l of this tile, over this wave's slice of K
+        float *mine = part + ((size_t)buf * nwaves + wave) * 256;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mine[r * 64 + lane] = acc[r];
+        __syncthreads();
+        if (wave == 0) {
+            float t[4];
+            const float *p = part + (size_t)buf * nwaves * 256;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) t[r] = p[r * 64 + lane];
+            for (int w2 = 1; w2 < nwaves; ++w2)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) t[r] += p[w2 * 256 + r * 64 + lane];
+            const int orow = tile * 16 + row_l;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = 4 * kb + r;
+                if (m < M && orow < N) out[(size_t)m * N + orow] = (uint16_t)f32_to_bf16_bits(t[r]);
+            }
+        }
+        // the other half of `part` takes the next tile: wave 0 reaches that tile's barrier
+        // only after it has read this half
+        buf ^= 1;
+    }
+}
+
+constexpr int kMaxDevices = 16;
+bool g_lin_ready[kMaxDevices];
+int g_lin_cus[kMaxDevices];
+int g_lin_lds[kMaxDevices];
+
 int g_rows_per_wave = 0;  // 0 = heuristic; set through bonsai_decode_set_tuning
 
 int rows_per_wave(int M) {
@@ -629,4 +734,50 @@ extern "C" int bonsai_draft_chain(const void *logits, int rows, int ld, int voca
     if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
     hipLaunchKernelGGL(draft_accept_kernel, dim3(1), dim3(64), 0, st, conf, rows, threshold, accept);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" int bonsai_bf16_linear(const void *x, const void *w, void *out, int M, int N, int K,
+                                  void *stream) {
+    if (!x || !w || !out) return BONSAI_DECODE_ERR_ARG;
+    if (M < 1 || M > BONSAI_MAX_WIDTH || N < 1 || K < 64 || K % 64 != 0) return BONSAI_DECODE_ERR_ARG;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
+    if (!g_lin_ready[dev]) {
+        int cus = 0, lds = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+            return BONSAI_DECODE_ERR_LAUNCH;
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(bf16_linear_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+            return BONSAI_DECODE_ERR_LAUNCH;
+        g_lin_cus[dev] = cus > 0 ? cus : 1;
+        g_lin_lds[dev] = lds;
+        g_lin_ready[dev] = true;
+    }
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return BONSAI_DECODE_ERR_ARG;
+    const int nwaves = K % 512 == 0 ? 8 : (K % 256 == 0 ? 4 : (K % 128 == 0 ? 2 : 1));
+    const int ntiles = (N + 15) / 16;
+    // token rows per launch: up to 16, fewer when that many rows of K do not fit in LDS
+    const size_t fixed = lin_lds_bytes(0, K, nwaves);
+    if (fixed + (size_t)(2 * K + 16) > (size_t)g_lin_lds[dev]) return BONSAI_DECODE_ERR_ARG;
+    int mt_max = (int)(((size_t)g_lin_lds[dev] - fixed) / (size_t)(2 * K + 16));
+    mt_max = mt_max < kLinTokens ? mt_max : kLinTokens;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (int m0 = 0; m0 < M; m0 += mt_max) {
+        const int mt = M - m0 < mt_max ? M - m0 : mt_max;
+        const size_t lds = lin_lds_bytes(mt, K, nwaves);
+        int per_cu = (int)((size_t)g_lin_lds[dev] / lds);
+        const int by_waves = 32 / nwaves;
+        per_cu = per_cu < by_waves ? per_cu : by_waves;
+        per_cu = per_cu < 1 ? 1 : per_cu;
+        const long want = (long)g_lin_cus[dev] * per_cu;
+        const int grid = (int)(ntiles < want ? ntiles : want);
+        hipLaunchKernelGGL(bf16_linear_kernel, dim3(grid), dim3(nwaves * 64), lds, st,
+                           static_cast<const uint16_t *>(x) + (size_t)m0 * K,
+                           static_cast<const uint16_t *>(w),
+                           static_cast<uint16_t *>(out) + (size_t)m0 * N, mt, N, K, nwaves, ntiles,
+                           grid);
+        if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
+    }
+    return BONSAI_DECODE_OK;
 }

@@ -1,7 +1,8 @@
-"""End-to-end decode throughput of a random-init packed-ternary model on one MI355X.
+"""End-to-end decode throughput of a random-init packed low-bit model on one MI355X.
 
     python -m bitmtp_amd.decode_bench --model 1.7b            # 256-token prompt, 512 new
     python -m bitmtp_amd.decode_bench --model 4b --prompt 512 --new 1024
+    python -m bitmtp_amd.decode_bench --model 4b --kind q1    # sign weights, bf16 lm_head
 
 Reports tokens/s by the reference's timing contract (``timed_decode_tokens /
 decode_time``, prefill and the first token excluded; src/bonsai_sft/gpu/fast_generate.py:
@@ -29,11 +30,12 @@ MODELS = {"1.7b": qwen3_1p7b_args, "4b": qwen3_4b_args}
 
 def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens: int = 512,
                      seed: int = 2, repeats: int = 2, device: str = "cuda:0",
-                     n_layers: int = 0) -> dict:
+                     n_layers: int = 0, kernel_kind: str = "t2g128", head_kind=None) -> dict:
     over = {"n_layers": n_layers} if n_layers else {}
+    over["kernel_kind"] = kernel_kind
     args = MODELS[model_name](**over)
     t0 = time.time()
-    model = BonsaiDecoder.random_init(args, seed=seed, device=device)
+    model = BonsaiDecoder.random_init(args, seed=seed, device=device, head_kind=head_kind)
     atlas = GraphAtlas(model, threshold=0.9)
     torch.cuda.synchronize()
     init_s = time.time() - t0
@@ -64,8 +66,10 @@ def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens
 
     hy_keys = ("committed_per_iter", "n_conf_path", "n_verify_path", "accept_rate")
     res = {
-        "model": f"random-init Qwen3-{model_name}-shaped T2-g128, {args.n_layers} layers, "
-                 f"dim {args.dim}, vocab {args.vocab_size}, packed T2 head",
+        "model": f"random-init Qwen3-{model_name}-shaped "
+                 f"{'T2-g128' if kernel_kind == 't2g128' else 'Q1-g128'}, {args.n_layers} layers, "
+                 f"dim {args.dim}, vocab {args.vocab_size}, "
+                 f"{ {'t2': 'packed T2', 'q1': 'packed Q1', 'bf16': 'bf16'}[model.head_kind] } head",
         "prompt_tokens": prompt_len, "new_tokens": new_tokens, "block_size": args.block_size,
         "weight_bytes_per_step": model.weight_bytes_per_step(),
         "init_s": round(init_s, 1),
@@ -88,9 +92,13 @@ def main() -> None:
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--repeats", type=int, default=2)
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = model's)")
+    ap.add_argument("--kind", choices=("t2g128", "q1"), default="t2g128",
+                    help="backbone weights: ternary T2-g128 or sign Q1-g128")
+    ap.add_argument("--head", choices=("t2", "q1", "bf16"), default=None,
+                    help="output projection (default: packed T2 for t2g128, bf16 for q1)")
     a = ap.parse_args()
     print(json.dumps(run_decode_bench(a.model, a.prompt, a.new, a.seed, a.repeats,
-                                      n_layers=a.layers)))
+                                      n_layers=a.layers, kernel_kind=a.kind, head_kind=a.head)))
 
 
 if __name__ == "__main__":

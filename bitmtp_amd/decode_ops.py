@@ -48,6 +48,8 @@ def load_decode_kernel() -> None:
     lib.bonsai_kv_commit.restype = ci
     lib.bonsai_draft_chain.argtypes = [vp, ci, ci, ci, cf, vp, vp, vp, vp]
     lib.bonsai_draft_chain.restype = ci
+    lib.bonsai_bf16_linear.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+    lib.bonsai_bf16_linear.restype = ci
     _lib = lib
 
 
@@ -181,3 +183,25 @@ def draft_chain(logits: torch.Tensor, vocab: int, threshold: float, tokens: torc
                                              _ptr(tokens), _ptr(conf), _ptr(accept),
                                              _stream(logits.device))
     _need(rc == 0, f"bonsai_draft_chain failed with status {rc}")
+
+
+def bf16_linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out = x @ w.T`` for a few bf16 rows ``x [M, K]`` and a bf16 matrix ``w [N, K]`` with
+    fp32 accumulation: the bf16 lm_head of a sign-weight backbone (reference: ``_lm_head``
+    with precision "bf16", model.py:1296).  ``out`` bf16 ``[M, N]`` is allocated when absent."""
+    _check(x, torch.bfloat16, "x")
+    _check(w, torch.bfloat16, "w")
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M, K] and w [N, K] must share K")
+    m, k = x.shape
+    n = w.shape[0]
+    _need(1 <= m <= MAX_WIDTH, f"bf16_linear takes 1..{MAX_WIDTH} rows")
+    _need(k % 64 == 0 and k >= 64, "K must be a multiple of 64")
+    if out is None:
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=x.device)
+    else:
+        _check(out, torch.bfloat16, "out")
+        _need(out.numel() >= m * n, "out too small")
+    with torch.cuda.device(x.device):
+        rc = decode_lib().bonsai_bf16_linear(_ptr(x), _ptr(w), _ptr(out), m, n, k, _stream(x.device))
+    _need(rc == 0, f"bonsai_bf16_linear failed with status {rc}")
+    return out

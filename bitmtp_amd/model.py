@@ -128,8 +128,9 @@ def rope_tables(args: ModelArgs, max_positions: int, device) -> Tuple[torch.Tens
 # ---------------------------------------------------------------------------
 @dataclass
 class PackedLinear:
-    weight: torch.Tensor        # int8 [N, K/4]
+    weight: torch.Tensor        # int8 [N, K/4] (ternary, bits = 2) or [N, K/8] (sign, bits = 1)
     weight_scale: torch.Tensor  # bf16 [N, K/128]
+    bits: int = 2
 
     @property
     def out_features(self) -> int:
@@ -137,7 +138,17 @@ class PackedLinear:
 
     @property
     def in_features(self) -> int:
-        return self.weight.shape[1] * 4
+        return self.weight.shape[1] * (8 // self.bits)
+
+
+def kind_bits(kernel_kind: str) -> int:
+    """Weight bits of a backbone kind: the reference's ``kernel_kind`` is "t2g128" (ternary)
+    or "q1" (sign weights), model.py:709."""
+    if kernel_kind == "t2g128":
+        return 2
+    if kernel_kind == "q1":
+        return 1
+    raise ValueError(f"unknown kernel_kind {kernel_kind!r} (expected 't2g128' or 'q1')")
 
 
 @dataclass
@@ -154,12 +165,16 @@ class LayerWeights:
     k_norm: torch.Tensor                    # bf16 [128]
 
 
-def _random_packed(n: int, k: int, gen: torch.Generator, device) -> PackedLinear:
-    """i.i.d. ternary codes (p = 1/3 each) and log-normal(-4, 0.5) group scales."""
-    codes = torch.randint(1, 4, (n, k), generator=gen, device=device, dtype=torch.uint8)
-    packed = _pack_fields(codes, 2)
+def _random_packed(n: int, k: int, gen: torch.Generator, device, bits: int = 2) -> PackedLinear:
+    """i.i.d. ternary codes (p = 1/3 each) or sign bits (p = 1/2) and log-normal(-4, 0.5)
+    group scales."""
+    if bits == 2:
+        codes = torch.randint(1, 4, (n, k), generator=gen, device=device, dtype=torch.uint8)
+    else:
+        codes = torch.randint(0, 2, (n, k), generator=gen, device=device, dtype=torch.uint8)
+    packed = _pack_fields(codes, bits)
     scale = torch.exp(torch.randn((n, k // GROUP_SIZE), generator=gen, device=device) * 0.5 - 4.0)
-    return PackedLinear(packed, scale.to(torch.bfloat16).contiguous())
+    return PackedLinear(packed, scale.to(torch.bfloat16).contiguous(), bits)
 
 
 def head_rows_for(vocab: int) -> int:
@@ -169,51 +184,89 @@ def head_rows_for(vocab: int) -> int:
 
 
 class BonsaiDecoder:
-    """Weights of a packed-ternary decoder plus its step enqueue function."""
+    """Weights of a packed low-bit decoder plus its step enqueue function.
+
+    ``head`` is the packed output projection (ternary for a "t2g128" backbone, as the
+    reference's graphs use, fast_runtime.py:115-118; sign-packed W1A8 for "q1" when asked for,
+    model.py:1262-1267), or None: then the logits come from the bf16 matrix ``head_bf16``
+    ``[vocab, dim]`` (the tied embedding unless given), which is what the reference's graphs
+    do for a "q1" backbone (fast_runtime.py:175-178)."""
 
     def __init__(self, args: ModelArgs, layers: List[LayerWeights], embed: torch.Tensor,
-                 norm: torch.Tensor, head: PackedLinear):
+                 norm: torch.Tensor, head: Optional[PackedLinear],
+                 head_bf16: Optional[torch.Tensor] = None):
         if args.head_dim != HEAD_DIM:
             raise ValueError("only head_dim 128 is supported")
-        if args.kernel_kind != "t2g128":
-            raise ValueError("the decode harness covers the ternary t2g128 backbone")
+        bits = kind_bits(args.kernel_kind)
         if args.dim % GROUP_SIZE or args.ffn_dim % GROUP_SIZE or args.q_dim % GROUP_SIZE:
             raise ValueError("dim, ffn_dim and n_heads*head_dim must be multiples of 128")
+        for lw in layers:
+            for p in (lw.wqkv, lw.wo, lw.w_gu, lw.w_down):
+                if p.bits != bits:
+                    raise ValueError(f"a {args.kernel_kind!r} backbone takes {bits}-bit layers")
         self.args = args
         self.layers = layers
         self.embed = embed          # bf16 [vocab, dim]
         self.norm = norm            # bf16 [dim]
-        self.head = head            # packed [head_rows, dim/4]
+        self.head = head            # packed [head_rows, dim*bits/8] or None
         self.device = embed.device
-        self.head_rows = head.out_features
+        if head is None:
+            w = embed if head_bf16 is None else head_bf16
+            if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != args.dim \
+                    or w.shape[0] < args.vocab_size:
+                raise ValueError("the bf16 head must be bf16 [>= vocab, dim]")
+            if w.shape[0] % 8:  # the logits' leading dimension must be a multiple of 8
+                padded = torch.zeros(-(-w.shape[0] // 8) * 8, args.dim, dtype=w.dtype, device=w.device)
+                padded[: w.shape[0]].copy_(w)
+                w = padded
+            self.head_bf16 = w.contiguous()
+            self.head_rows = self.head_bf16.shape[0]
+        else:
+            self.head_bf16 = None
+            self.head_rows = head.out_features
+
+    @property
+    def head_kind(self) -> str:
+        if self.head is None:
+            return "bf16"
+        return "t2" if self.head.bits == 2 else "q1"
 
     # -- construction --------------------------------------------------------
     @classmethod
-    def random_init(cls, args: ModelArgs, seed: int = 0, device="cuda") -> "BonsaiDecoder":
-        """Random ternary weights; the embedding is the dequantised tied head, as in a
-        converted checkpoint whose tied projection sits on the ternary grid
-        (reference: ``prepare_t2_lm_head``, model.py:1222-1243)."""
+    def random_init(cls, args: ModelArgs, seed: int = 0, device="cuda",
+                    head_kind: Optional[str] = None) -> "BonsaiDecoder":
+        """Random low-bit weights; the embedding is the dequantised tied head, as in a
+        converted checkpoint whose tied projection sits on the weight grid (reference:
+        ``prepare_t2_lm_head`` / ``prepare_q1_lm_head``, model.py:1196-1243).  ``head_kind``
+        "t2", "q1" or "bf16"; by default what the reference's graphs use for the backbone:
+        the packed ternary head for "t2g128", the bf16 matrix for "q1"."""
         device = torch.device(device)
         gen = torch.Generator(device=device)
         gen.manual_seed(seed)
+        bits = kind_bits(args.kernel_kind)
+        if head_kind is None:
+            head_kind = "t2" if bits == 2 else "bf16"
+        if head_kind not in ("t2", "q1", "bf16"):
+            raise ValueError(f"unknown head_kind {head_kind!r}")
         layers = []
         for _ in range(args.n_layers):
             def ln(n):
                 return (1.0 + 0.1 * torch.randn(n, generator=gen, device=device)).to(torch.bfloat16)
             layers.append(LayerWeights(
-                wqkv=_random_packed(args.q_dim + 2 * args.kv_dim, args.dim, gen, device),
-                wo=_random_packed(args.dim, args.q_dim, gen, device),
-                w_gu=_random_packed(2 * args.ffn_dim, args.dim, gen, device),
-                w_down=_random_packed(args.dim, args.ffn_dim, gen, device),
+                wqkv=_random_packed(args.q_dim + 2 * args.kv_dim, args.dim, gen, device, bits),
+                wo=_random_packed(args.dim, args.q_dim, gen, device, bits),
+                w_gu=_random_packed(2 * args.ffn_dim, args.dim, gen, device, bits),
+                w_down=_random_packed(args.dim, args.ffn_dim, gen, device, bits),
                 input_layernorm=ln(args.dim), post_attention_layernorm=ln(args.dim),
                 q_norm=ln(HEAD_DIM), k_norm=ln(HEAD_DIM)))
         rows = head_rows_for(args.vocab_size)
-        head = _random_packed(rows, args.dim, gen, device)
+        head = _random_packed(rows, args.dim, gen, device, 1 if head_kind == "q1" else
+                              (2 if head_kind == "t2" else bits))
         if rows > args.vocab_size:
             head.weight_scale[args.vocab_size:] = 0
-        embed = dequantize_t2(head)[: args.vocab_size].contiguous()
+        embed = dequantize_packed(head)[: args.vocab_size].contiguous()
         norm = (1.0 + 0.1 * torch.randn(args.dim, generator=gen, device=device)).to(torch.bfloat16)
-        return cls(args, layers, embed, norm, head)
+        return cls(args, layers, embed, norm, None if head_kind == "bf16" else head)
 
     def weight_bytes_per_step(self) -> int:
         """Packed weight + scale bytes one replay streams (head included)."""
@@ -221,17 +274,28 @@ class BonsaiDecoder:
         for lw in self.layers:
             for p in (lw.wqkv, lw.wo, lw.w_gu, lw.w_down):
                 total += p.weight.numel() + 2 * p.weight_scale.numel()
+        if self.head is None:
+            return total + 2 * self.head_bf16.numel()
         return total + self.head.weight.numel() + 2 * self.head.weight_scale.numel()
 
 
-def dequantize_t2(p: PackedLinear) -> torch.Tensor:
-    """bf16 [N, K] = (code - 2) * group scale (reference: ``_unpack_to_bf16``, model.py:641-647)."""
+def dequantize_packed(p: PackedLinear) -> torch.Tensor:
+    """bf16 [N, K]: ``(code - 2) * scale`` for ternary weights, ``(2 bit - 1) * scale`` for
+    sign weights (reference: ``_unpack_to_bf16``, model.py:641-647 and :585-593)."""
     b = p.weight.view(torch.uint8)
-    shifts = torch.arange(0, 8, 2, device=b.device, dtype=torch.uint8)
-    q = ((b.unsqueeze(-1) >> shifts) & 3).to(torch.int8) - 2
+    if p.bits == 2:
+        shifts = torch.arange(0, 8, 2, device=b.device, dtype=torch.uint8)
+        q = ((b.unsqueeze(-1) >> shifts) & 3).to(torch.int8) - 2
+    else:
+        shifts = torch.arange(0, 8, 1, device=b.device, dtype=torch.uint8)
+        q = ((b.unsqueeze(-1) >> shifts) & 1).to(torch.int8) * 2 - 1
     n = b.shape[0]
     q = q.view(n, -1, GROUP_SIZE).to(torch.bfloat16)
     return (q * p.weight_scale.unsqueeze(-1)).view(n, -1)
+
+
+def dequantize_t2(p: PackedLinear) -> torch.Tensor:
+    return dequantize_packed(p)
 
 
 # ---------------------------------------------------------------------------
@@ -266,6 +330,7 @@ class Workspace:
         self.h_last = buf((m_max, args.dim), bf)
         self.l_q = buf((m_max, args.dim), i8)
         self.l_s = buf((m_max,), f32)
+        self.l_n = buf((m_max, args.dim), bf)
         self.logits = buf((m_max, head_rows), bf)
 
 
@@ -322,11 +387,11 @@ def _vp(t: torch.Tensor) -> ctypes.c_void_p:
 
 def _gemv(a_q: torch.Tensor, a_s: torch.Tensor, w: PackedLinear, out: torch.Tensor, m: int,
           stream: ctypes.c_void_p) -> None:
-    rc = ops.t2_lib().t2g128_gemv_ex(_vp(a_q), _vp(w.weight), _vp(out), _vp(a_s),
-                                     _vp(w.weight_scale), m, w.out_features, w.in_features,
-                                     ops.OUT_BF16, ops.SCALE_BF16, stream)
+    fn = ops.t2_lib().t2g128_gemv_ex if w.bits == 2 else ops.q1_lib().q1g128_gemv_ex
+    rc = fn(_vp(a_q), _vp(w.weight), _vp(out), _vp(a_s), _vp(w.weight_scale), m, w.out_features,
+            w.in_features, ops.OUT_BF16, ops.SCALE_BF16, stream)
     if rc != 0:
-        raise RuntimeError(f"t2g128_gemv_ex failed with status {rc}")
+        raise RuntimeError(f"{'t2g128' if w.bits == 2 else 'q1g128'}_gemv_ex failed with status {rc}")
 
 
 def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tensor, sigma: int,
@@ -383,10 +448,20 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
         _gemv(ws.i_q, ws.i_s, lw.w_down, ws.ffn_out, M, stream)
 
     rows = logits_end - logits_start
-    check(actq.bonsai_add_rmsnorm_quant_int8(_vp(ws.ffn_out[logits_start:]), _vp(h_cur[logits_start:]),
-                                             _vp(model.norm), eps, _vp(ws.h_last), _vp(ws.l_q),
-                                             _vp(ws.l_s), rows, dim, stream),
-          "bonsai_add_rmsnorm_quant_int8")
-    _gemv(ws.l_q, ws.l_s, model.head, ws.logits, rows, stream)
+    if model.head is None:
+        # bf16 projection of the normalised rows (reference: model.py:1401-1403 with
+        # lm_head_precision "bf16")
+        check(actq.bonsai_add_rmsnorm_bf16(_vp(ws.ffn_out[logits_start:]), _vp(h_cur[logits_start:]),
+                                           _vp(model.norm), eps, _vp(ws.h_last), _vp(ws.l_n),
+                                           rows, dim, stream),
+              "bonsai_add_rmsnorm_bf16")
+        decode_ops.bf16_linear(ws.l_n[:rows], model.head_bf16, ws.logits)
+    else:
+        check(actq.bonsai_add_rmsnorm_quant_int8(_vp(ws.ffn_out[logits_start:]),
+                                                 _vp(h_cur[logits_start:]), _vp(model.norm), eps,
+                                                 _vp(ws.h_last), _vp(ws.l_q), _vp(ws.l_s), rows,
+                                                 dim, stream),
+              "bonsai_add_rmsnorm_quant_int8")
+        _gemv(ws.l_q, ws.l_s, model.head, ws.logits, rows, stream)
     decode_ops.draft_chain(ws.logits[:rows], args.vocab_size, threshold, io.tokens_out, io.conf,
                            io.accept)

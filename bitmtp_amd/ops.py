@@ -110,6 +110,8 @@ def load_actq_kernel() -> None:
     lib.bonsai_rmsnorm_quant_int8.restype = ci
     lib.bonsai_add_rmsnorm_quant_int8.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, vp, ci, ci, vp]
     lib.bonsai_add_rmsnorm_quant_int8.restype = ci
+    lib.bonsai_add_rmsnorm_bf16.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, ci, ci, vp]
+    lib.bonsai_add_rmsnorm_bf16.restype = ci
     lib.bonsai_silu_mul_quant_int8.argtypes = [vp, vp, vp, ci, ci, vp]
     lib.bonsai_silu_mul_quant_int8.restype = ci
     _actq_lib = lib
@@ -355,6 +357,27 @@ def fused_add_norm_quant(x: torch.Tensor, residual: torch.Tensor, w: torch.Tenso
     if rc != 0:
         raise RuntimeError(f"fused_add_norm_quant: native launch failed with status {rc}")
     return h, q, s
+
+
+def add_rmsnorm(x: torch.Tensor, residual: Optional[torch.Tensor], w: torch.Tensor,
+                eps: float) -> torch.Tensor:
+    """``RMSNorm(x + residual) * w`` in bf16 without quantisation (``residual`` may be None):
+    the final norm in front of a bf16 output projection (reference: model.py:1401-1402,
+    ``RMSNorm.forward`` model.py:290-295)."""
+    ts = (x, w) if residual is None else (x, residual, w)
+    _check_bf16_rows("add_rmsnorm", *ts)
+    k = x.shape[-1]
+    if (residual is not None and residual.shape != x.shape) or w.shape != (k,) or k % 8 != 0:
+        raise RuntimeError("add_rmsnorm: shape mismatch or K not a multiple of 8")
+    m = x.numel() // k
+    n = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = actq_lib().bonsai_add_rmsnorm_bf16(_ptr(x), _ptr(residual) if residual is not None
+                                                else ctypes.c_void_p(0), _ptr(w), float(eps),
+                                                ctypes.c_void_p(0), _ptr(n), m, k, _stream(x.device))
+    if rc != 0:
+        raise RuntimeError(f"add_rmsnorm: native launch failed with status {rc}")
+    return n
 
 
 def silu_mul_quant(gate_up: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -103,6 +103,16 @@ int bonsai_kv_commit(void *kv, int n_layers, int n_kv, int slots, int src_slot, 
 int bonsai_draft_chain(const void *logits, int rows, int ld, int vocab, float threshold,
                        int32_t *tokens, float *conf, int32_t *accept, void *stream);
 
+/* bf16 output projection of a sign-weight (Q1) backbone, whose graphs keep the tied lm_head
+ * in bf16: logits = F.linear(h, W) (`_lm_head`, precision "bf16",
+ * src/bonsai_sft/gpu/model.py:1296; chosen in src/bonsai_sft/gpu/fast_runtime.py:175-178).
+ *   x bf16 [M, K], w bf16 [N, K] row-major, out bf16 [M, N]; M <= BONSAI_MAX_WIDTH, K % 64 == 0
+ * fp32 accumulation in a fixed order (k ascending inside a slice of K, slices left to
+ * right), one RNE rounding to bf16.  The reference's library GEMM fixes no order, so the
+ * result is compared with an fp32 matmul to one bf16 step.  The first call on a device sets
+ * a function attribute: make it outside stream capture. */
+int bonsai_bf16_linear(const void *x, const void *w, void *out, int M, int N, int K, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

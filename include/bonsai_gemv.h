@@ -134,6 +134,14 @@ int bonsai_rmsnorm_quant_int8(const void *x, const void *w, float eps, int8_t *q
 int bonsai_add_rmsnorm_quant_int8(const void *x, const void *residual, const void *w, float eps,
                                   void *h_out, int8_t *q, float *s, int M, int K, void *stream);
 
+/* Residual add + RMSNorm without quantisation: the final `h = h + ffn_out; norm(h[rows])`
+ * in front of a bf16 output projection (src/bonsai_sft/gpu/model.py:1401-1402 with
+ * `RMSNorm.forward`, model.py:290-295).  n_out = bf16(w * bf16(fp32(h) * rsqrt(var + eps)))
+ * [M,K], h = bf16(x + residual), or h = x when residual is NULL; h_out [M,K] receives h
+ * when it and residual are not NULL. */
+int bonsai_add_rmsnorm_bf16(const void *x, const void *residual, const void *w, float eps,
+                            void *h_out, void *n_out, int M, int K, void *stream);
+
 /* SiLU(gate) * up + quantisation of the merged gate/up GEMV output
  * (src/bonsai_sft/gpu/model.py:1058-1061): gate_up bf16 [M, 2F] with the gate in
  * columns [0,F) and up in [F,2F); inner = bf16(bf16(silu(gate)) * up); q int8

@@ -315,28 +315,47 @@ static void quant_row(const float *nf, int8_t *q, float *s, int K) {
 
 /* _fused_norm_quant / _fused_add_norm_quant.  X, RES (may be NULL), W are bf16 bit
  * patterns; H (may be NULL) receives bf16(x + residual).  K <= 65536. */
+static void rmsnorm_row(const uint16_t *x, const uint16_t *res, const uint16_t *W, float eps,
+                        uint16_t *hrow, float *nf, int K) {
+    static float h[65536];
+    for (int k = 0; k < K; ++k) {
+        float v = oracle_bf16_to_f32(x[k]);
+        if (res) {
+            volatile float sum = v + oracle_bf16_to_f32(res[k]);
+            v = bf16_round_f(sum);
+            if (hrow) hrow[k] = oracle_f32_to_bf16(v);
+        }
+        h[k] = v;
+    }
+    float var = (float)sumsq_kernel_order(h, K) / (float)K;
+    volatile float root = sqrtf(var + eps);
+    float rs = 1.0f / root;
+    for (int k = 0; k < K; ++k) {
+        volatile float t = h[k] * rs;
+        volatile float u = oracle_bf16_to_f32(W[k]) * bf16_round_f(t);
+        nf[k] = bf16_round_f(u);
+    }
+}
+
 void oracle_rmsnorm_quant(const uint16_t *X, const uint16_t *RES, const uint16_t *W, float eps,
                           uint16_t *H, int8_t *Q, float *S, int M, int K) {
-    static float h[65536], nf[65536];
+    static float nf[65536];
     for (int m = 0; m < M; ++m) {
-        for (int k = 0; k < K; ++k) {
-            float v = oracle_bf16_to_f32(X[(size_t)m * K + k]);
-            if (RES) {
-                volatile float sum = v + oracle_bf16_to_f32(RES[(size_t)m * K + k]);
-                v = bf16_round_f(sum);
-                if (H) H[(size_t)m * K + k] = oracle_f32_to_bf16(v);
-            }
-            h[k] = v;
-        }
-        float var = (float)sumsq_kernel_order(h, K) / (float)K;
-        volatile float root = sqrtf(var + eps);
-        float rs = 1.0f / root;
-        for (int k = 0; k < K; ++k) {
-            volatile float t = h[k] * rs;
-            volatile float u = oracle_bf16_to_f32(W[k]) * bf16_round_f(t);
-            nf[k] = bf16_round_f(u);
-        }
+        rmsnorm_row(X + (size_t)m * K, RES ? RES + (size_t)m * K : NULL, W, eps,
+                    H ? H + (size_t)m * K : NULL, nf, K);
         quant_row(nf, Q + (size_t)m * K, S + m, K);
+    }
+}
+
+/* The same norm without the quantisation: RMSNorm.forward on h = x (+ residual)
+ * (src/bonsai_sft/gpu/model.py:290-295, 1401-1402).  NOUT receives bf16(w * bf16(h * rs)). */
+void oracle_rmsnorm_bf16(const uint16_t *X, const uint16_t *RES, const uint16_t *W, float eps,
+                         uint16_t *H, uint16_t *NOUT, int M, int K) {
+    static float nf[65536];
+    for (int m = 0; m < M; ++m) {
+        rmsnorm_row(X + (size_t)m * K, RES ? RES + (size_t)m * K : NULL, W, eps,
+                    H ? H + (size_t)m * K : NULL, nf, K);
+        for (int k = 0; k < K; ++k) NOUT[(size_t)m * K + k] = oracle_f32_to_bf16(nf[k]);
     }
 }
 
@@ -355,4 +374,4 @@ void oracle_silu_mul_quant(const uint16_t *GU, int8_t *Q, float *S, int M, int F
     }
 }
 
-int oracle_abi_version(void) { return 2; }
+int oracle_abi_version(void) { return 3; }

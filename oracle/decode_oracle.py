@@ -176,7 +176,10 @@ def decode_step(weights: dict, kv_k: np.ndarray, kv_v: np.ndarray, tokens, posit
     """One graph forward (model.py:1386-1403) on the CPU.
 
     ``weights``: ``embed`` (bf16 bits [vocab, dim]), ``norm``, ``head`` = (packed uint8, scale
-    bits), ``cos``/``sin`` bits, ``eps``, ``n_heads``, ``n_kv``, and ``layers`` = list of dicts
+    bits) with ``head_bits`` (default ``bits``) or, for the bf16 projection of a sign-weight
+    backbone (model.py:1296), ``head_bf16`` = bf16 bits [rows, dim]; ``bits`` = 2 (ternary,
+    default) or 1 (sign) for the layers; ``cos``/``sin`` bits, ``eps``, ``n_heads``, ``n_kv``,
+    and ``layers`` = list of dicts
     with ``wqkv``/``wo``/``w_gu``/``w_down`` (packed, scale bits), ``input_layernorm``,
     ``post_attention_layernorm``, ``q_norm``, ``k_norm`` (bf16 bits).
     ``kv_k``/``kv_v``: bf16 bits [n_layers, n_kv, slots, 128], updated in place at
@@ -187,8 +190,10 @@ def decode_step(weights: dict, kv_k: np.ndarray, kv_v: np.ndarray, tokens, posit
     M = len(tokens)
     scale = 1.0 / np.sqrt(HEAD_DIM)
 
-    def gemv(q8, s, w):
-        _, y_bits = O.c_gemv(q8, w[0], s, w[1], 2)
+    bits = weights.get("bits", 2)
+
+    def gemv(q8, s, w, b=bits):
+        _, y_bits = O.c_gemv(q8, w[0], s, w[1], b)
         return y_bits
 
     h = weights["embed"][np.asarray(tokens)]
@@ -212,6 +217,14 @@ def decode_step(weights: dict, kv_k: np.ndarray, kv_v: np.ndarray, tokens, posit
         gu = gemv(f_q, f_s, lw["w_gu"])
         i_q, i_s = O.c_silu_mul_quant(gu)
         ffn_out = gemv(i_q, i_s, lw["w_down"])
+    if weights.get("head_bf16") is not None:
+        n_bits, _ = O.c_rmsnorm(ffn_out[logits_start:logits_end], weights["norm"], eps,
+                                residual_bits=h[logits_start:logits_end])
+        # fp32 accumulation of exact bf16 products; float64 here, the order is the library's
+        # in the reference, so callers compare with a tolerance of one bf16 step
+        y = O.bf16_bits_to_f32(n_bits).astype(np.float64) @ \
+            O.bf16_bits_to_f32(weights["head_bf16"]).astype(np.float64).T
+        return O.f32_to_bf16_bits(y.astype(np.float32))
     l_q, l_s, _ = O.c_rmsnorm_quant(ffn_out[logits_start:logits_end], weights["norm"], eps,
                                     residual_bits=h[logits_start:logits_end])
-    return gemv(l_q, l_s, weights["head"])
+    return gemv(l_q, l_s, weights["head"], weights.get("head_bits", bits))

@@ -55,6 +55,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_gemv.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
         L.oracle_rmsnorm_quant.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, vp, ci, ci]
         L.oracle_rmsnorm_quant.restype = None
+        L.oracle_rmsnorm_bf16.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, ci, ci]
+        L.oracle_rmsnorm_bf16.restype = None
         L.oracle_silu_mul_quant.argtypes = [vp, vp, vp, ci, ci]
         L.oracle_silu_mul_quant.restype = None
         L.oracle_f32_to_bf16.argtypes = [ctypes.c_float]
@@ -147,6 +149,21 @@ def c_rmsnorm_quant(x_bits, w_bits, eps: float, residual_bits=None):
     H = np.empty((M, K), dtype=np.uint16)
     lib().oracle_rmsnorm_quant(_p(X), _p(R), _p(W), eps, _p(H), _p(Q), _p(S), M, K)
     return Q, S, H
+
+
+def c_rmsnorm(x_bits, w_bits, eps: float, residual_bits=None):
+    """RMSNorm without quantisation: returns (normed bf16 bits [M,K], h bf16 bits or None)."""
+    X = _c(x_bits, np.uint16)
+    W = _c(w_bits, np.uint16)
+    M, K = X.shape
+    N = np.empty((M, K), dtype=np.uint16)
+    if residual_bits is None:
+        lib().oracle_rmsnorm_bf16(_p(X), None, _p(W), eps, None, _p(N), M, K)
+        return N, None
+    R = _c(residual_bits, np.uint16)
+    H = np.empty((M, K), dtype=np.uint16)
+    lib().oracle_rmsnorm_bf16(_p(X), _p(R), _p(W), eps, _p(H), _p(N), M, K)
+    return N, H
 
 
 def c_silu_mul_quant(gu_bits):

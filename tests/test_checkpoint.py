@@ -331,3 +331,39 @@ def test_converted_checkpoint_loads_and_decodes(tmp_path):
     ar, _ = ar_generate(atlas, prompt, max_gen_len=20)
     hy, st = hybrid_generate(atlas, prompt, max_gen_len=20, exact_m1_verify=True)
     assert len(ar) == 20 and hy == ar
+
+
+@pytest.mark.gpu
+def test_converted_q1_checkpoint_loads_and_decodes(tmp_path):
+    """A sign-weight checkpoint decodes with 1-bit layers and the bf16 tied output projection
+    (fast_runtime.py:175-178); exact verification reproduces the AR tokens."""
+    from bitmtp_amd.generate import ar_generate, hybrid_generate
+    from bitmtp_amd.model import dequantize_packed
+    from bitmtp_amd.runtime import GraphAtlas
+    src, out = tmp_path / "hf", tmp_path / "converted"
+    src.mkdir()
+    cfg = dict(BASE_CONFIG, hidden_size=512, intermediate_size=1024, num_attention_heads=4,
+               num_key_value_heads=2, num_hidden_layers=2, vocab_size=1000, block_size=8,
+               text_mask_token_id=999)
+    (src / "config.json").write_text(json.dumps(cfg))
+    gen = torch.Generator().manual_seed(9)
+
+    def fill(shape):
+        if len(shape) == 1:
+            return 1.0 + 0.1 * torch.randn(*shape, generator=gen)
+        return torch.randn(*shape, generator=gen) * 0.02
+    save_file(ones_weights(cfg, fill=fill), str(src / "model.safetensors"))
+    C.convert(str(src), str(out), quant="q1")
+    model = C.load_decoder(str(out), device="cuda:0")
+    frozen = torch.load(out / "model_state_fp16.pt", weights_only=True)
+    assert model.head_kind == "bf16" and model.head_rows == 1000
+    lw = model.layers[0]
+    assert lw.wqkv.bits == 1 and lw.wqkv.in_features == 512
+    want = torch.cat([frozen[f"layers.0.attention.{p}_proj.weight"] for p in "qkv"], dim=0)
+    assert torch.equal(dequantize_packed(lw.wqkv).cpu(), want)
+    assert torch.equal(model.head_bf16.cpu(), frozen["embed_tokens.weight"])
+    atlas = GraphAtlas(model, segment_ladder=(128,))
+    prompt = list(range(5, 31))
+    ar, _ = ar_generate(atlas, prompt, max_gen_len=16)
+    hy, _ = hybrid_generate(atlas, prompt, max_gen_len=16, exact_m1_verify=True)
+    assert len(ar) == 16 and hy == ar

@@ -174,6 +174,31 @@ def test_draft_chain_kernel(DO, rows, vocab, ld):
     assert accept.cpu().tolist() == [wn, rows]
 
 
+# ---------------------------------------------------------------- bf16 output projection
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 512), (9, 4099, 2048), (16, 1536, 2560), (17, 300, 64),
+                                   (32, 129, 128), (3, 7, 320), (5, 151936, 2048)])
+def test_bf16_linear_against_fp32_matmul(M, N, K):
+    """fp32 accumulation of exact bf16 products, one rounding: the bf16 result is within one
+    bf16 step of the rounded float64 product (the reference's library GEMM fixes no order)."""
+    from bitmtp_amd import decode_ops
+    rng = np.random.default_rng(M * 131 + N + K)
+    x = _rand_bf16(rng, (M, K), 1.0).to(DEV)
+    w = _rand_bf16(rng, (N, K), 0.05).to(DEV)
+    print(f"[case] bf16_linear M={M} N={N} K={K}", flush=True)
+    got = decode_ops.bf16_linear(x, w)
+    torch.cuda.synchronize()
+    want = (x.double() @ w.double().T)
+    want_b = want.to(torch.bfloat16)
+    d = np.abs(bf16_ordinal(bf16_bits(got)) - bf16_ordinal(bf16_bits(want_b)))
+    small = (want.abs() < 1e-3 * want.abs().max()).cpu().numpy()
+    assert d[~small].max() <= 1
+    assert (d[~small] != 0).mean() < 0.05
+    assert (got.double() - want).abs().max().item() <= 1e-2 * want.abs().max().item()
+    # a preallocated output with a wider leading dimension is rejected, wrong K as well
+    with pytest.raises(RuntimeError):
+        decode_ops.bf16_linear(x, w[:, : K - 64].contiguous() if K > 64 else w[:, :32].contiguous())
+
+
 # ---------------------------------------------------------------- whole step and loops
 def _tiny_args(**over):
     from bitmtp_amd.model import ModelArgs
@@ -196,8 +221,11 @@ def _oracle_weights(model, atlas):
     def pl(p):
         return (p.weight.cpu().numpy().view(np.uint8), bf16_bits(p.weight_scale))
     a = model.args
+    head = {"head": pl(model.head), "head_bits": model.head.bits} if model.head is not None \
+        else {"head_bf16": bf16_bits(model.head_bf16)}
     return {
-        "embed": bf16_bits(model.embed), "norm": bf16_bits(model.norm), "head": pl(model.head),
+        "embed": bf16_bits(model.embed), "norm": bf16_bits(model.norm), **head,
+        "bits": model.layers[0].wqkv.bits,
         "cos": bf16_bits(atlas.rope[0]), "sin": bf16_bits(atlas.rope[1]), "eps": a.norm_eps,
         "n_heads": a.n_heads, "n_kv": a.n_kv_heads,
         "layers": [{
@@ -385,3 +413,70 @@ def test_replay_argument_checks(tiny):
         atlas.get_graph(4, 64, "draft")
     with pytest.raises(KeyError):
         atlas.kv(100)
+
+
+# ---------------------------------------------------------------- sign-weight (Q1) backbone
+@pytest.fixture(scope="module", params=["bf16", "q1"])
+def tiny_q1(request):
+    """A "q1" backbone with the bf16 output projection the reference's graphs use for it
+    (fast_runtime.py:175-178) and with the sign-packed W1A8 projection (model.py:1262-1267)."""
+    from bitmtp_amd.model import BonsaiDecoder
+    from bitmtp_amd.runtime import GraphAtlas
+    model = BonsaiDecoder.random_init(_tiny_args(kernel_kind="q1"), seed=13, device=DEV,
+                                      head_kind=request.param)
+    assert model.head_kind == request.param and model.layers[0].wo.bits == 1
+    atlas = GraphAtlas(model, segment_ladder=(64, 256), threshold=0.9)
+    return model, atlas
+
+
+@pytest.mark.parametrize("role,M,n_pend", [("ar", 1, 0), ("verify", 9, 0), ("draft", 12, 3)])
+def test_q1_step_against_cpu_composition(DO, tiny_q1, role, M, n_pend):
+    from bitmtp_amd import runtime
+    from oracle import oracle as O
+    model, atlas = tiny_q1
+    sigma, cache_len = 64, 17
+    rng = np.random.default_rng(100 + M)
+    kv = atlas.kv(sigma)
+    kv.copy_(_rand_bf16(rng, tuple(kv.shape), 0.5).to(DEV))
+    kv_bits = bf16_bits(kv)
+    tokens = rng.integers(0, model.args.vocab_size, M).tolist()
+    positions = [cache_len + i for i in range(M)]
+    g = atlas.get_graph(M, sigma, role)
+    print(f"q1 step case head={model.head_kind} {role} M={M}", flush=True)
+    atlas.replay(g, tokens, positions, cache_len, n_pend=n_pend)
+    toks, conf, accept = atlas.read_outputs(g)
+    rows = g.logits_end - g.logits_start
+    got = atlas.workspace.logits[:rows, : model.args.vocab_size].float().cpu().numpy()
+    desc = runtime.step_descriptor(role, M, atlas.D, cache_len, n_pend)
+    vis = runtime.dense_visibility(desc, M, sigma)
+    kk, vv = kv_bits[0].copy(), kv_bits[1].copy()
+    want_bits = DO.decode_step(_oracle_weights(model, atlas), kk, vv, tokens, positions, vis, sigma,
+                               g.logits_start, g.logits_end)
+    want = O.bf16_bits_to_f32(want_bits)[:, : model.args.vocab_size]
+    assert np.abs(got - want).max() <= 6e-2 * np.abs(want).max()
+    wt, wc, wn = DO.draft_chain(got, atlas.threshold)
+    assert toks.tolist() == wt.tolist() and accept == wn
+    np.testing.assert_allclose(conf, wc, rtol=2e-3, atol=1e-6)
+
+
+def test_q1_hybrid_with_exact_verification_reproduces_ar(tiny_q1):
+    from bitmtp_amd import generate
+    model, atlas = tiny_q1
+    rng = np.random.default_rng(23)
+    prompt = rng.integers(0, 1000, 29).tolist()
+    ar, _ = generate.ar_generate(atlas, prompt, max_gen_len=32)
+    hy, st = generate.hybrid_generate(atlas, prompt, max_gen_len=32, exact_m1_verify=True)
+    assert len(ar) == 32 and hy == ar
+    assert st["draft_iters"] == st["n_conf_path"] + st["n_verify_path"]
+    # replays of a captured bf16-head graph are repeatable (no stale state in the graph)
+    again, _ = generate.ar_generate(atlas, prompt, max_gen_len=32)
+    assert again == ar
+
+
+def test_decoder_rejects_mixed_weight_kinds():
+    from bitmtp_amd.model import BonsaiDecoder
+    model = BonsaiDecoder.random_init(_tiny_args(), seed=3, device=DEV)
+    with pytest.raises(ValueError):
+        BonsaiDecoder(_tiny_args(kernel_kind="q1"), model.layers, model.embed, model.norm, None)
+    with pytest.raises(ValueError):
+        BonsaiDecoder.random_init(_tiny_args(kernel_kind="w4"), seed=3, device=DEV)

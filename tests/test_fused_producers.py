@@ -54,6 +54,25 @@ def test_oracle_norm_quant_matches_torch(oracle, M, K):
     assert np.array_equal(s, st.numpy().reshape(-1)) and np.array_equal(q, qt.numpy())
 
 
+@pytest.mark.parametrize("M,K", [(1, 128), (3, 2048), (9, 2560)])
+def test_oracle_norm_without_quant_matches_torch(oracle, M, K):
+    """The norm-only form is RMSNorm.forward (model.py:290-295) on x or on x + residual."""
+    x, r, w = make_inputs(7 * K + M, M, K)
+    eps = 1e-6
+
+    def torch_norm(h):
+        hf = h.float()
+        return w * (hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + eps)).to(h.dtype)
+    n, h = oracle.c_rmsnorm(bits(x), bits(w), eps)
+    assert h is None and np.array_equal(n, bits(torch_norm(x)))
+    n, h = oracle.c_rmsnorm(bits(x), bits(w), eps, bits(r))
+    assert np.array_equal(h, bits(x + r)) and np.array_equal(n, bits(torch_norm(x + r)))
+    # known answer: x = 2, w = 0.5, eps = 0 -> rms 2, normed 0.5 everywhere
+    n, _ = oracle.c_rmsnorm(bits(torch.full((1, 256), 2.0, dtype=torch.bfloat16)),
+                            bits(torch.full((256,), 0.5, dtype=torch.bfloat16)), 0.0)
+    assert np.all(n == 0x3F00)
+
+
 def test_oracle_norm_quant_known_answer(oracle):
     """x = 2 everywhere, w = 0.5, eps = 0: rms = 2, normed = 0.5, s = 254, q = 127."""
     x = torch.full((1, 256), 2.0, dtype=torch.bfloat16)
@@ -111,6 +130,24 @@ def test_hip_norm_quant_bit_exact(oracle, M, K):
     q_ref, s_ref, h_ref = oracle.c_rmsnorm_quant(bits(x), bits(w), eps, bits(r))
     assert np.array_equal(bits(h.cpu()), h_ref)
     assert np.array_equal(s.cpu().numpy().reshape(-1), s_ref) and np.array_equal(q.cpu().numpy(), q_ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K", [(1, 128), (1, 2048), (9, 2048), (17, 2560), (2, 9728)])
+def test_hip_norm_without_quant_bit_exact(oracle, M, K):
+    import bitmtp_amd as ops
+    x, r, w = make_inputs(K * 5 + M, M, K)
+    eps = 1e-6
+    dev = "cuda:0"
+    print(f"[case] add_rmsnorm M={M} K={K}", flush=True)
+    n = ops.add_rmsnorm(x.to(dev), None, w.to(dev), eps)
+    n_ref, _ = oracle.c_rmsnorm(bits(x), bits(w), eps)
+    assert n.shape == x.shape and np.array_equal(bits(n.cpu()), n_ref)
+    n = ops.add_rmsnorm(x.to(dev), r.to(dev), w.to(dev), eps)
+    n_ref, _ = oracle.c_rmsnorm(bits(x), bits(w), eps, bits(r))
+    assert np.array_equal(bits(n.cpu()), n_ref)
+    with pytest.raises(RuntimeError):
+        ops.add_rmsnorm(x.to(dev), r[:, :-8].contiguous().to(dev), w.to(dev), eps)
 
 
 @pytest.mark.gpu
