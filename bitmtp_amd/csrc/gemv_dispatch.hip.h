@@ -1,14 +1,16 @@
 // Entry-point logic shared by libbonsai_t2.so and libbonsai_q1.so: argument
 // checks, one-time device set-up and the choice among the kernels.  Measured on
-// MI355X: the dot4 kernel (packed_gemv.hip.h) is fastest up to four tokens on
-// layer-sized matrices, the int8 matrix-core kernel (gemv_mfma.hip.h) from five
-// tokens on and from two tokens on for very long matrices (the lm_head).  The
-// FP4 x FP8 matrix-core kernel (gemv_fp4.hip.h) needs fewer VALU operations per
-// byte but its FP8 staging and deeper register use make it no faster yet; it
-// runs only when selected with the tuning call.  Shapes the matrix-core kernels
-// do not take (K not a multiple of 512, unaligned operands, token tiles that do
-// not fit in LDS) go to the dot4 kernel.  Replaces the if-chain over registered (M, N, K) of the
-// reference (src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:94-148).
+// MI355X: the dot4 kernel (packed_gemv.hip.h) is fastest for one and two tokens
+// on layer-sized matrices; from three tokens on (from two for very long matrices,
+// the lm_head) the int8 matrix-core kernels (gemv_mfma.hip.h) win: the one that
+// loads the activations straight as operands up to 16384 rows, the one that
+// stages them in LDS once per workgroup above.  The FP4 x FP8 matrix-core kernel
+// (gemv_fp4.hip.h) needs fewer VALU operations per byte but its FP8 staging and
+// deeper register use make it no faster yet; it runs only when selected with the
+// tuning call.  Shapes the matrix-core kernels do not take (K not a multiple of
+// 512, unaligned operands, token tiles that do not fit in LDS) go to the dot4
+// kernel.  Replaces the if-chain over registered (M, N, K) of the reference
+// (src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:94-148).
 #ifndef BONSAI_GEMV_DISPATCH_HIP_H
 #define BONSAI_GEMV_DISPATCH_HIP_H
 
@@ -39,7 +41,7 @@ int init_all_kernels() {
     return 0;
 }
 
-// Launches one of the two matrix-core kernels.  Returns -1 when the shape does not
+// Launches one of the matrix-core kernels (engine 1 staged int8, 2 FP4 x FP8, 3 direct int8).  Returns -1 when the shape does not
 // fit (the caller falls back), 0 on success, 2 on a launch error.  `single_tile`
 // refuses shapes whose tokens would need more than ceil(M/16) token tiles, i.e.
 // a second pass over the weights.
