@@ -156,12 +156,40 @@ def cpu_baseline(budget_s: float):
         t_used += time.perf_counter() - t0
         reps += 1
     total_bytes = reps * len(WIDTHS) * LAYER_BYTES
-    return {
+    res = {
         "value": round(total_bytes / t_used / 1e9, 3), "unit": "GB/s", "cores": threads,
         "kind": "port",
         "sample": f"{reps} x (one 1.7B-shaped layer, 7 T2 projections at widths 1,4,8) in "
                   f"{t_used:.1f} s with the C oracle, OpenMP over rows",
     }
+    # Second figure: the only statement of the op the reference can run on a CPU,
+    # F.linear(dequantised activations, dequantised weights) in bf16
+    # (src/bonsai_sft/gpu/model.py:646-656), with this build's own PyTorch.
+    import torch
+    import torch.nn.functional as F
+    dense = []
+    for p in problems:
+        w = O.np_unpack(p["B"], 2).astype(np.float32).reshape(p["B"].shape[0], -1, O.GROUP)
+        w = (w * O.bf16_bits_to_f32(p["ws"])[:, :, None]).reshape(p["B"].shape[0], -1)
+        x = p["A"].astype(np.float32) / p["s"].reshape(-1, 1)
+        dense.append((torch.from_numpy(x).to(torch.bfloat16), torch.from_numpy(w).to(torch.bfloat16)))
+    reps2, t2 = 0, 0.0
+    with torch.no_grad():
+        for x, w in dense:   # untimed first pass
+            F.linear(x, w)
+        while t2 < budget_s / 3 and reps2 < 200:
+            t0 = time.perf_counter()
+            for x, w in dense:
+                F.linear(x, w)
+            t2 += time.perf_counter() - t0
+            reps2 += 1
+    res["torch_cpu_f_linear"] = {
+        "value": round(reps2 * len(WIDTHS) * LAYER_BYTES / t2 / 1e9, 3), "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "sample": f"{reps2} x the same 21 products as bf16 F.linear on dequantised operands in "
+                  f"{t2:.1f} s (same algorithmic bytes counted)",
+    }
+    return res
 
 
 def main() -> int:

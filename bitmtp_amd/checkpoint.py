@@ -24,7 +24,7 @@ import json
 import math
 import os
 from pathlib import Path
-from typing import Dict, List, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -387,13 +387,14 @@ def load_packed_state(ckpt_dir: str) -> Tuple[object, Dict[str, torch.Tensor]]:
     return args, sd
 
 
-def load_decoder(ckpt_dir: str, device="cuda"):
+def load_decoder(ckpt_dir: str, device="cuda", head_kind: Optional[str] = None):
     """Packed checkpoint -> ``BonsaiDecoder`` with q|k|v and gate|up merged along the output
     rows (``prepare_merged_weights``, model.py:931-956,1042-1051).  A ternary checkpoint gets
     the tied head packed on its ternary grid, padded to whole 128-row tiles
     (``prepare_t2_lm_head``, model.py:1222-1243); a sign-weight ("q1") checkpoint keeps the
     output projection in bf16 (the tied embedding, or ``lm_head.weight`` when untied), as the
-    reference's graphs do (fast_runtime.py:175-178)."""
+    reference's graphs do (fast_runtime.py:175-178); ``head_kind="q1"`` packs it to sign bits
+    instead (``prepare_q1_lm_head``, model.py:1196-1220)."""
     from .model import BonsaiDecoder, LayerWeights, PackedLinear, head_rows_for, kind_bits
     args, sd = load_packed_state(ckpt_dir)
     dev = torch.device(device)
@@ -417,7 +418,19 @@ def load_decoder(ckpt_dir: str, device="cuda"):
             post_attention_layernorm=sd[f"layers.{i}.post_attention_layernorm.weight"].to(dev),
             q_norm=sd[a + "q_norm.weight"].to(dev), k_norm=sd[a + "k_norm.weight"].to(dev)))
     embed = sd["embed_tokens.weight"].to(dev).contiguous()
+    if head_kind not in (None, "t2", "q1", "bf16") or (bits == 2 and head_kind not in (None, "t2")):
+        raise ValueError(f"head_kind {head_kind!r} does not fit a {args.kernel_kind!r} checkpoint")
+    if bits == 1 and head_kind == "q1":
+        src = embed if args.tie_word_embeddings else sd["lm_head.weight"].to(dev)
+        rows = head_rows_for(args.vocab_size)
+        padded = torch.zeros(rows, args.dim, dtype=torch.bfloat16, device=dev)
+        padded[: args.vocab_size].copy_(src)
+        head_w, head_s = pack_q1_g128(padded)
+        return BonsaiDecoder(args, layers, embed, sd["norm.weight"].to(dev),
+                             PackedLinear(head_w, head_s, 1))
     if bits == 1:
+        if head_kind == "t2":
+            raise ValueError("a 'q1' checkpoint takes head_kind 'bf16' or 'q1'")
         head_bf16 = None
         if not args.tie_word_embeddings:
             if "lm_head.weight" not in sd:

@@ -51,9 +51,10 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
                        int scale_kind, int lds_limit, hipStream_t stream) {
     const MfmaTuning &tu = mfma_tuning<BITS>();
     const bool fp4 = engine == 2, direct = engine == 3;
+    int nw = 4;  // waves per workgroup; eight only for the direct kernel on long rows
     auto lds_for = [&](int ri, int mt) {
         return fp4 ? fp4_lds_for<BITS>(ri, mt, K)
-                   : (direct ? mfma_direct_lds_for<BITS>(ri) : mfma_lds_for<BITS>(ri, mt, K));
+                   : (direct ? mfma_direct_lds_for<BITS>(ri, nw) : mfma_lds_for<BITS>(ri, mt, K));
     };
     int ntok_tiles = (M + kMfmaTokens - 1) / kMfmaTokens;
     int mt = (M + ntok_tiles - 1) / ntok_tiles;
@@ -69,18 +70,22 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
     int R = tu.row_tiles;
     const int ntiles = K / 512;
     if (ks == 0) {
-        if (direct)  // no staging to amortise: split K as far as it goes
-            ks = ntiles >= 4 ? 4 : (ntiles >= 2 ? 2 : 1);
+        if (direct)  // no staging to amortise: split K as far as it goes; eight waves per
+                     // workgroup only while that leaves at most about one workgroup per CU
+            ks = (ntiles >= 8 && N <= 4096) ? 8 : (ntiles >= 4 ? 4 : (ntiles >= 2 ? 2 : 1));
         else
             ks = (N <= 4096 && ntiles >= 4) ? 4 : ((N <= 16384 && ntiles >= 2) ? 2 : 1);
     }
-    if (ks != 1 && ks != 2 && ks != 4) ks = 1;
+    if (ks != 1 && ks != 2 && ks != 4 && !(ks == 8 && direct)) ks = 1;
     // slices may be uneven (tile t goes to slice floor-partition): every wave still reaches the
     // single barrier after its K loop; an empty slice is never scheduled
     if (ks > ntiles) ks = 1;
+    if (ks == 8) nw = 8;
     if (R == 0) {
-        const long wgs1 = ((long)N + 16 * (4 / ks) - 1) / (16 * (4 / ks));  // workgroups at R = 1
+        const long wgs1 = ((long)N + 16 * (nw / ks) - 1) / (16 * (nw / ks));  // workgroups at R = 1
         R = wgs1 >= 8192 ? 4 : (wgs1 >= 2048 ? 2 : 1);
+        // long rows walked tile after tile: two row tiles per wave double the bytes in flight
+        if (direct && R == 1 && ntiles / ks >= 4 && wgs1 >= 512) R = 2;
     }
     int ri = R >= 4 ? 2 : (R >= 2 ? 1 : 0);
     while (ri > 0 && lds_for(ri, mt) > (size_t)lds_limit) --ri;
@@ -106,19 +111,20 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
     args.N = N;
     args.K = K;
     args.mt = mt;
-    args.ks_log2 = ks == 4 ? 2 : (ks == 2 ? 1 : 0);
+    args.ks_log2 = ks == 8 ? 3 : (ks == 4 ? 2 : (ks == 2 ? 1 : 0));
     args.out_f32 = out_kind == OUT_F32 ? 1 : 0;
     args.passes = passes;
     const int per_token = fp4 ? K / 32 : K / mfma_quarter_bytes<BITS>();  // staging tasks per token
     args.div_magic = (uint32_t)(0x100000000ull / (uint64_t)per_token) + 1u;
 
-    const int rows_per_wg = 16 * R * (4 / ks) * passes;
+    const int rows_per_wg = 16 * R * (nw / ks) * passes;
     const int grid_x = (N + rows_per_wg - 1) / rows_per_wg;
     const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
     const MfmaKernelFn fn = fp4 ? fp4_table<BITS>().fn[ri][variant]
-                                : (direct ? mfma_direct_table<BITS>().fn[ri][variant]
+                                : (direct ? (nw == 8 ? mfma_direct8_table<BITS>().fn[ri][variant]
+                                                     : mfma_direct_table<BITS>().fn[ri][variant])
                                           : mfma_table<BITS>().fn[ri][variant]);
-    hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(kMfmaThreads, 1, 1), lds_for(ri, mt),
+    hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(nw * 64, 1, 1), lds_for(ri, mt),
                        stream, args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
                        args.mt, args.ks_log2, args.out_f32, args.passes, args.div_magic);
     return hipGetLastError() == hipSuccess ? 0 : 2;

@@ -316,13 +316,15 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel
 // the accumulator layout).  No workgroup barrier before the K loop and no LDS for
 // activations: the kernel is one memory round trip plus the K loop long.
 // ---------------------------------------------------------------------------
-template <int BITS, int R>
+// NW = waves per workgroup: four, or eight for long rows (K >= 4096), where a wave would
+// otherwise walk through several K tiles one memory round trip after the other.
+template <int BITS, int R, int NW = 4>
 __host__ __device__ inline size_t mfma_direct_lds_bytes() {
-    return (size_t)4 * mfma_wave_tile_bytes<BITS, R>() + (size_t)4 * R * 4 * 64 * 4;
+    return (size_t)NW * mfma_wave_tile_bytes<BITS, R>() + (size_t)NW * R * 4 * 64 * 4;
 }
 
-template <int BITS, int R, bool G32, bool SF16>
-__global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_direct_kernel
+template <int BITS, int R, bool G32, bool SF16, int NW = 4>
+__global__ void __launch_bounds__(NW * 64) gemv_mfma_direct_kernel
 (const int8_t *pA, const uint8_t *pB, void *pout, const float *ps, const uint16_t *pws, int pM,
  int pN, int pK, int pmt, int pks_log2, int pout_f32, int ppasses, uint32_t pdiv_magic) {
     // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
@@ -339,7 +341,7 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_direct_kernel
     const int ks = 1 << a.ks_log2;
     const int kslice = wave & (ks - 1);
     const int rw = wave >> a.ks_log2;
-    const int rws = 4 >> a.ks_log2;
+    const int rws = NW >> a.ks_log2;
     const int m0 = blockIdx.y * a.mt;
     const int mt = (M - m0) < a.mt ? (M - m0) : a.mt;
     const int pass_rows = rws * 16 * R;
@@ -347,7 +349,7 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_direct_kernel
 
     unsigned char *tiles = smem;
     unsigned char *wt = tiles + (size_t)wave * mfma_wave_tile_bytes<BITS, R>();
-    float *red = reinterpret_cast<float *>(tiles + (size_t)4 * mfma_wave_tile_bytes<BITS, R>());
+    float *red = reinterpret_cast<float *>(tiles + (size_t)NW * mfma_wave_tile_bytes<BITS, R>());
 
     const int ntiles = G / kMfmaGroupsPerTile;
     const int t_begin = (int)(((long)ntiles * kslice) >> a.ks_log2);
@@ -546,7 +548,7 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_direct_kernel
 struct MfmaTuning {
     int min_width = 0;   // smallest M sent to this kernel; 0 = built-in default
     int row_tiles = 0;   // R: 1, 2 or 4; 0 = heuristic
-    int k_split = 0;     // waves along K: 1, 2 or 4; 0 = heuristic
+    int k_split = 0;     // waves along K: 1, 2, 4 (or 8: direct kernel, eight waves); 0 = heuristic
     int passes = 0;      // row blocks per workgroup; 0 = heuristic
     int engine = 0;      // 0 = choose, 1 = int8 MFMA (staged), 2 = FP4 x FP8 MFMA, 3 = int8 MFMA (direct)
 };
@@ -596,8 +598,31 @@ const MfmaTable<BITS> &mfma_direct_table() {
     return t;
 }
 
+// the eight-wave form of the direct kernel
 template <int BITS>
-size_t mfma_direct_lds_for(int ri) {
+const MfmaTable<BITS> &mfma_direct8_table() {
+    static const MfmaTable<BITS> t = [] {
+        MfmaTable<BITS> x{};
+        x.fn[0][0] = gemv_mfma_direct_kernel<BITS, 1, false, false, 8>;
+        x.fn[0][1] = gemv_mfma_direct_kernel<BITS, 1, false, true, 8>;
+        x.fn[0][2] = gemv_mfma_direct_kernel<BITS, 1, true, false, 8>;
+        x.fn[1][0] = gemv_mfma_direct_kernel<BITS, 2, false, false, 8>;
+        x.fn[1][1] = gemv_mfma_direct_kernel<BITS, 2, false, true, 8>;
+        x.fn[1][2] = gemv_mfma_direct_kernel<BITS, 2, true, false, 8>;
+        x.fn[2][0] = gemv_mfma_direct_kernel<BITS, 4, false, false, 8>;
+        x.fn[2][1] = gemv_mfma_direct_kernel<BITS, 4, false, true, 8>;
+        x.fn[2][2] = gemv_mfma_direct_kernel<BITS, 4, true, false, 8>;
+        return x;
+    }();
+    return t;
+}
+
+template <int BITS>
+size_t mfma_direct_lds_for(int ri, int nw = 4) {
+    if (nw == 8)
+        return ri == 0 ? mfma_direct_lds_bytes<BITS, 1, 8>()
+                       : (ri == 1 ? mfma_direct_lds_bytes<BITS, 2, 8>()
+                                  : mfma_direct_lds_bytes<BITS, 4, 8>());
     return ri == 0 ? mfma_direct_lds_bytes<BITS, 1>()
                    : (ri == 1 ? mfma_direct_lds_bytes<BITS, 2>() : mfma_direct_lds_bytes<BITS, 4>());
 }
@@ -610,7 +635,8 @@ MfmaTuning &mfma_tuning() {
 
 template <int BITS>
 int mfma_init_device(int max_lds) {
-    const MfmaTable<BITS> *tables[2] = {&mfma_table<BITS>(), &mfma_direct_table<BITS>()};
+    const MfmaTable<BITS> *tables[3] = {&mfma_table<BITS>(), &mfma_direct_table<BITS>(),
+                                        &mfma_direct8_table<BITS>()};
     for (const MfmaTable<BITS> *t : tables)
         for (int r = 0; r < 3; ++r)
             for (int v = 0; v < 3; ++v)

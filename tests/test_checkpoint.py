@@ -367,3 +367,11 @@ def test_converted_q1_checkpoint_loads_and_decodes(tmp_path):
     ar, _ = ar_generate(atlas, prompt, max_gen_len=16)
     hy, _ = hybrid_generate(atlas, prompt, max_gen_len=16, exact_m1_verify=True)
     assert len(ar) == 16 and hy == ar
+    # the sign-packed head: scale = bf16(mean |w|) per group, bit = (w >= 0), 24 zero pad rows
+    packed = C.load_decoder(str(out), device="cuda:0", head_kind="q1")
+    assert packed.head_kind == "q1" and packed.head_rows == 1024
+    w = frozen["embed_tokens.weight"].float().view(1000, 4, 128)
+    assert torch.equal(packed.head.weight_scale[:1000].cpu(), w.abs().mean(-1).to(torch.bfloat16))
+    assert torch.all(packed.head.weight_scale[1000:] == 0)
+    with pytest.raises(ValueError):
+        C.load_decoder(str(out), device="cuda:0", head_kind="t2")
