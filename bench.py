@@ -304,12 +304,17 @@ def main() -> int:
 
     # The other half of the headline metric: end-to-end decode tokens/s of the random-init
     # 1.7B-shaped model (configs[2]), AR and D8 hybrid, by the reference's timing contract.
-    decode = None
+    decode = decode_bf16 = None
     if not args.no_decode:
         del run, pool, graph
         torch.cuda.empty_cache()
         from bitmtp_amd.decode_bench import run_decode_bench
         decode = run_decode_bench("1.7b", prompt_len=256, new_tokens=512, repeats=1)
+        torch.cuda.empty_cache()
+        # the same model with the output projection kept in bf16 (622 MB per step instead of
+        # the 83 MB packed head the reference's graphs use for a ternary backbone)
+        decode_bf16 = run_decode_bench("1.7b", prompt_len=256, new_tokens=512, repeats=1,
+                                       head_kind="bf16")
 
     cpu = cpu_baseline(args.cpu_seconds) if args.cpu_seconds > 0 else None
 
@@ -328,6 +333,7 @@ def main() -> int:
             "timing": "one HIP graph of all steps, HIP events on the launch stream, best of 3 replays",
             "lm_head_151936x2048": head,
             "decode_1p7b_d8": decode,
+            "decode_1p7b_d8_bf16_lm_head": decode_bf16,
         },
         "roofline": roofline,
         "cpu_baseline": cpu,

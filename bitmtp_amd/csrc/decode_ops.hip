@@ -9,6 +9,8 @@
 //   draft_rows_kernel / draft_accept_kernel   argmax + confidence chain
 //                         (src/bonsai_sft/gpu/fast_generate.py:111-130)
 //   bf16_linear_kernel    bf16 lm_head of a sign-weight backbone (model.py:1296)
+//   fp8_quant_rows_kernel / fp8_linear_kernel   E4M3 draft projection (model.py:1168-1194,
+//                         1268-1275)
 //
 // Attention is HBM/L2-bound integer-free fp work: per layer it reads
 // 2 * n_kv * (cache_len + M) * 256 bytes of KV once per query-head group.  The mask
@@ -590,6 +592,162 @@ bool g_lin_ready[kMaxDevices];
 int g_lin_cus[kMaxDevices];
 int g_lin_lds[kMaxDevices];
 
+// ---------------------------------------------------------------------------
+// FP8 (E4M3, OCP "fn") draft projection of the reference (`prepare_fp8_lm_head` and
+// `_lm_head` with precision "fp8", src/bonsai_sft/gpu/model.py:1168-1194,1268-1275): the
+// rows are quantised with ONE scale for all of them, amax / 448 evaluated in bf16 like the
+// reference's tensor expression, and multiplied with a per-tensor-scaled E4M3 weight matrix.
+// ---------------------------------------------------------------------------
+constexpr int kFp8Threads = 1024;
+
+// fp32 -> E4M3 (bias 7, no infinities, 0x7f = NaN), round to nearest even, subnormals kept;
+// magnitudes that round above 448 give NaN like torch's cast (they cannot occur after the
+// division by the row scale)
+__device__ __forceinline__ uint32_t f32_to_e4m3fn(float f) {
+    const uint32_t u = __float_as_uint(f);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    const uint32_t au = u & 0x7fffffffu;
+    if (au > 0x7f800000u) return sign | 0x7fu;  // NaN
+    const float af = __uint_as_float(au);
+    if (af > 464.0f) return sign | 0x7fu;        // beyond the rounding range of 448 (464 ties to 448)
+    if (af < 0.015625f) {                        // below 2^-6: multiples of 2^-9
+        const float q = rintf(af * 512.0f);      // round half to even
+        return sign | (uint32_t)q;               // q == 8 is the smallest normal, same code
+    }
+    // normal: keep 3 mantissa bits, RNE on the 20 dropped ones
+    uint32_t r = au + 0x7ffffu + ((au >> 20) & 1u);
+    const uint32_t exp = (r >> 23) - 127u + 7u;
+    const uint32_t man = (r >> 20) & 7u;
+    return sign | (exp << 3) | man;
+}
+
+// x bf16 [M, K] -> q E4M3 [M, K], scale[0] = fp32(bf16(max(bf16(amax / 448), 1e-12)));
+// q = e4m3(bf16(fp32(x) / scale)).  One workgroup: M * K is a few rows of the hidden size.
+__global__ void __launch_bounds__(kFp8Threads)
+fp8_quant_rows_kernel(const uint16_t *x, uint8_t *q, float *scale, int total) {
+    __shared__ float wave_max[kFp8Threads / 64];
+    const int tid = threadIdx.x;
+    const int nvec = total / 8;
+    float amax = 0.0f;
+    for (int v = tid; v < nvec; v += kFp8Threads) {
+        const uint4 raw = reinterpret_cast<const uint4 *>(x)[v];
+        const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            amax = fmaxf(amax, fabsf(bf16_bits_to_f32(d[i] & 0xffffu)));
+            amax = fmaxf(amax, fabsf(__uint_as_float(d[i] & 0xffff0000u)));
+        }
+    }
+    amax = bonsai_wave::max64(amax);
+    if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+    __syncthreads();
+    float t = wave_max[0];
+    for (int w = 1; w < kFp8Threads / 64; ++w) t = fmaxf(t, wave_max[w]);
+    // bf16 arithmetic of the reference expression: (amax / 448).clamp_min(1e-12).float()
+    float sc = bf16_round(t / 448.0f);
+    sc = fmaxf(sc, bf16_round(1e-12f));
+    if (tid == 0) scale[0] = sc;
+    for (int v = tid; v < nvec; v += kFp8Threads) {
+        const uint4 raw = reinterpret_cast<const uint4 *>(x)[v];
+        const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+        uint32_t o[2] = {0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = bf16_round(bf16_bits_to_f32(d[i] & 0xffffu) / sc);
+            const float hi = bf16_round(__uint_as_float(d[i] & 0xffff0000u) / sc);
+            o[i >> 1] |= (f32_to_e4m3fn(lo) | (f32_to_e4m3fn(hi) << 8)) << (16 * (i & 1));
+        }
+        reinterpret_cast<uint2 *>(q)[v] = make_uint2(o[0], o[1]);
+    }
+}
+
+__host__ __device__ inline size_t fp8_lin_lds_bytes(int M, int K, int nwaves) {
+    return (size_t)M * (K + 16) + (size_t)2 * nwaves * 256 * sizeof(float);
+}
+
+// out[m][n] = bf16( (sum_k x[m][k] * w[n][k]) * x_scale * w_scale ), E4M3 operands, fp32
+// accumulation.  Same structure as bf16_linear_kernel: tokens in LDS, the waves split K,
+// a lane streams 32 contiguous bytes (four K-blocks of 8) of its weight row per group of
+// four v_mfma_f32_16x16x32_fp8_fp8.
+__global__ void __launch_bounds__(kLinMaxWaves * 64)
+fp8_linear_kernel(const uint8_t *x, const float *x_scale, const uint8_t *w, float w_scale,
+                  uint16_t *out, int M, int N, int K, int nwaves, int ntiles, int grid) {
+    extern __shared__ __align__(16) unsigned char lin_smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pitch = K + 16;
+    float *part = reinterpret_cast<float *>(lin_smem + (size_t)M * pitch);
+
+    const int vec_per_row = K / 16;
+    for (int v = tid; v < M * vec_per_row; v += nwaves * 64) {
+        const int m = v / vec_per_row, c = v - m * vec_per_row;
+        *reinterpret_cast<uint4 *>(lin_smem + (size_t)m * pitch + (size_t)c * 16) =
+            reinterpret_cast<const uint4 *>(x + (size_t)m * K)[c];
+    }
+    __syncthreads();
+    const float scale = x_scale[0] * w_scale;
+
+    const int row_l = lane & 15, kb = lane >> 4;
+    const int ksl = K / nwaves;     // a multiple of 128
+    const int nblk = ksl / 128;
+    const int k_base = wave * ksl + 32 * kb;
+    const int tok = row_l < M ? row_l : M - 1;
+    const unsigned char *xl = lin_smem + (size_t)tok * pitch + k_base;
+    int buf = 0;
+    for (int tile = blockIdx.x; tile < ntiles; tile += grid) {
+        int row = tile * 16 + row_l;
+        row = row < N ? row : N - 1;
+        const uint4 *wl = reinterpret_cast<const uint4 *>(w + (size_t)row * K + k_base);
+        f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int p0 = 0; p0 < nblk; p0 += kLinUnroll) {
+            uint4 wr[kLinUnroll][2];
+#pragma unroll
+            for (int u = 0; u < kLinUnroll; ++u)
+                if (p0 + u < nblk) {
+                    wr[u][0] = wl[(p0 + u) * 8];
+                    wr[u][1] = wl[(p0 + u) * 8 + 1];
+                }
+#pragma unroll
+            for (int u = 0; u < kLinUnroll; ++u)
+                if (p0 + u < nblk) {
+                    const uint4 x0 = *reinterpret_cast<const uint4 *>(xl + (size_t)(p0 + u) * 128);
+                    const uint4 x1 = *reinterpret_cast<const uint4 *>(xl + (size_t)(p0 + u) * 128 + 16);
+                    const uint32_t xs[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                    const uint32_t ws[8] = {wr[u][0].x, wr[u][0].y, wr[u][0].z, wr[u][0].w,
+                                            wr[u][1].x, wr[u][1].y, wr[u][1].z, wr[u][1].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const long xa = (long)(((uint64_t)xs[2 * j + 1] << 32) | xs[2 * j]);
+                        const long wb = (long)(((uint64_t)ws[2 * j + 1] << 32) | ws[2 * j]);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(xa, wb, acc, 0, 0, 0);
+                    }
+                }
+        }
+        float *mine = part + ((size_t)buf * nwaves + wave) * 256;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mine[r * 64 + lane] = acc[r];
+        __syncthreads();
+        if (wave == 0) {
+            float t[4];
+            const float *p = part + (size_t)buf * nwaves * 256;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) t[r] = p[r * 64 + lane];
+            for (int w2 = 1; w2 < nwaves; ++w2)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) t[r] += p[w2 * 256 + r * 64 + lane];
+            const int orow = tile * 16 + row_l;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = 4 * kb + r;
+                if (m < M && orow < N)
+                    out[(size_t)m * N + orow] = (uint16_t)f32_to_bf16_bits(t[r] * scale);
+            }
+        }
+        buf ^= 1;
+    }
+}
+
+bool g_fp8_ready[kMaxDevices];
+
 int g_rows_per_wave = 0;  // 0 = heuristic; set through bonsai_decode_set_tuning
 
 int rows_per_wave(int M) {
@@ -775,6 +933,61 @@ extern "C" int bonsai_bf16_linear(const void *x, const void *w, void *out, int M
         hipLaunchKernelGGL(bf16_linear_kernel, dim3(grid), dim3(nwaves * 64), lds, st,
                            static_cast<const uint16_t *>(x) + (size_t)m0 * K,
                            static_cast<const uint16_t *>(w),
+                           static_cast<uint16_t *>(out) + (size_t)m0 * N, mt, N, K, nwaves, ntiles,
+                           grid);
+        if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
+    }
+    return BONSAI_DECODE_OK;
+}
+
+extern "C" int bonsai_fp8_quant_rows(const void *x, void *q, float *scale, int M, int K,
+                                     void *stream) {
+    if (!x || !q || !scale) return BONSAI_DECODE_ERR_ARG;
+    if (M < 1 || M > BONSAI_MAX_WIDTH || K < 8 || K % 8 != 0) return BONSAI_DECODE_ERR_ARG;
+    hipLaunchKernelGGL(fp8_quant_rows_kernel, dim3(1), dim3(kFp8Threads), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(x),
+                       static_cast<uint8_t *>(q), scale, M * K);
+    return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" int bonsai_fp8_linear(const void *x, const float *x_scale, const void *w, float w_scale,
+                                 void *out, int M, int N, int K, void *stream) {
+    if (!x || !x_scale || !w || !out) return BONSAI_DECODE_ERR_ARG;
+    if (M < 1 || M > BONSAI_MAX_WIDTH || N < 1 || K < 128 || K % 128 != 0) return BONSAI_DECODE_ERR_ARG;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return BONSAI_DECODE_ERR_ARG;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
+    if (!g_fp8_ready[dev]) {
+        int cus = 0, lds = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+            return BONSAI_DECODE_ERR_LAUNCH;
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(fp8_linear_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+            return BONSAI_DECODE_ERR_LAUNCH;
+        g_lin_cus[dev] = cus > 0 ? cus : 1;
+        g_lin_lds[dev] = lds;
+        g_fp8_ready[dev] = true;
+    }
+    const int nwaves = K % 1024 == 0 ? 8 : (K % 512 == 0 ? 4 : (K % 256 == 0 ? 2 : 1));
+    const int ntiles = (N + 15) / 16;
+    const size_t fixed = fp8_lin_lds_bytes(0, K, nwaves);
+    if (fixed + (size_t)(K + 16) > (size_t)g_lin_lds[dev]) return BONSAI_DECODE_ERR_ARG;
+    int mt_max = (int)(((size_t)g_lin_lds[dev] - fixed) / (size_t)(K + 16));
+    mt_max = mt_max < kLinTokens ? mt_max : kLinTokens;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (int m0 = 0; m0 < M; m0 += mt_max) {
+        const int mt = M - m0 < mt_max ? M - m0 : mt_max;
+        const size_t lds = fp8_lin_lds_bytes(mt, K, nwaves);
+        int per_cu = (int)((size_t)g_lin_lds[dev] / lds);
+        const int by_waves = 32 / nwaves;
+        per_cu = per_cu < by_waves ? per_cu : by_waves;
+        per_cu = per_cu < 1 ? 1 : per_cu;
+        const long want = (long)g_lin_cus[dev] * per_cu;
+        const int grid = (int)(ntiles < want ? ntiles : want);
+        hipLaunchKernelGGL(fp8_linear_kernel, dim3(grid), dim3(nwaves * 64), lds, st,
+                           static_cast<const uint8_t *>(x) + (size_t)m0 * K, x_scale,
+                           static_cast<const uint8_t *>(w), w_scale,
                            static_cast<uint16_t *>(out) + (size_t)m0 * N, mt, N, K, nwaves, ntiles,
                            grid);
         if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;

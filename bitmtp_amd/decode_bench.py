@@ -30,13 +30,18 @@ MODELS = {"1.7b": qwen3_1p7b_args, "4b": qwen3_4b_args}
 
 def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens: int = 512,
                      seed: int = 2, repeats: int = 2, device: str = "cuda:0",
-                     n_layers: int = 0, kernel_kind: str = "t2g128", head_kind=None) -> dict:
+                     n_layers: int = 0, kernel_kind: str = "t2g128", head_kind=None,
+                     draft_precision: str = "native") -> dict:
     over = {"n_layers": n_layers} if n_layers else {}
     over["kernel_kind"] = kernel_kind
     args = MODELS[model_name](**over)
     t0 = time.time()
     model = BonsaiDecoder.random_init(args, seed=seed, device=device, head_kind=head_kind)
-    atlas = GraphAtlas(model, threshold=0.9)
+    draft_kw = {"fp8": {"use_fp8_draft": True}, "bf16": {"use_bf16_draft": True},
+                "native": {}}[draft_precision]
+    roles = ("ar", "draft", "verify") + {"fp8": ("draft_fp8",), "bf16": ("draft_bf16",),
+                                         "native": ()}[draft_precision]
+    atlas = GraphAtlas(model, threshold=0.9, roles=roles)
     torch.cuda.synchronize()
     init_s = time.time() - t0
     rng = np.random.default_rng(seed)
@@ -52,9 +57,9 @@ def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens
 
     out_ar, st_ar = best(lambda: ar_generate(atlas, prompt, max_gen_len=new_tokens))
     out_hy, st_hy = best(lambda: hybrid_generate(atlas, prompt, threshold=0.9,
-                                                 max_gen_len=new_tokens))
+                                                 max_gen_len=new_tokens, **draft_kw))
     out_fc, st_fc = best(lambda: hybrid_generate(atlas, prompt, threshold=0.0, hybrid_m=1,
-                                                 max_gen_len=new_tokens))
+                                                 max_gen_len=new_tokens, **draft_kw))
 
     def line(st, extra=()):
         d = {"tokens_per_s": round(st["timed_decode_tokens"] / st["decode_time"], 1),
@@ -70,6 +75,7 @@ def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens
                  f"{'T2-g128' if kernel_kind == 't2g128' else 'Q1-g128'}, {args.n_layers} layers, "
                  f"dim {args.dim}, vocab {args.vocab_size}, "
                  f"{ {'t2': 'packed T2', 'q1': 'packed Q1', 'bf16': 'bf16'}[model.head_kind] } head",
+        "draft_projection": draft_precision,
         "prompt_tokens": prompt_len, "new_tokens": new_tokens, "block_size": args.block_size,
         "weight_bytes_per_step": model.weight_bytes_per_step(),
         "init_s": round(init_s, 1),
@@ -96,9 +102,13 @@ def main() -> None:
                     help="backbone weights: ternary T2-g128 or sign Q1-g128")
     ap.add_argument("--head", choices=("t2", "q1", "bf16"), default=None,
                     help="output projection (default: packed T2 for t2g128, bf16 for q1)")
+    ap.add_argument("--draft", choices=("native", "fp8", "bf16"), default="native",
+                    help="draft output projection: the backbone's own, or the FP8 / raw bf16 "
+                         "approximation (verification always uses the backbone's own)")
     a = ap.parse_args()
     print(json.dumps(run_decode_bench(a.model, a.prompt, a.new, a.seed, a.repeats,
-                                      n_layers=a.layers, kernel_kind=a.kind, head_kind=a.head)))
+                                      n_layers=a.layers, kernel_kind=a.kind, head_kind=a.head,
+                                      draft_precision=a.draft)))
 
 
 if __name__ == "__main__":

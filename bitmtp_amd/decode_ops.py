@@ -50,6 +50,10 @@ def load_decode_kernel() -> None:
     lib.bonsai_draft_chain.restype = ci
     lib.bonsai_bf16_linear.argtypes = [vp, vp, vp, ci, ci, ci, vp]
     lib.bonsai_bf16_linear.restype = ci
+    lib.bonsai_fp8_quant_rows.argtypes = [vp, vp, vp, ci, ci, vp]
+    lib.bonsai_fp8_quant_rows.restype = ci
+    lib.bonsai_fp8_linear.argtypes = [vp, vp, vp, cf, vp, ci, ci, ci, vp]
+    lib.bonsai_fp8_linear.restype = ci
     _lib = lib
 
 
@@ -204,4 +208,68 @@ def bf16_linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     with torch.cuda.device(x.device):
         rc = decode_lib().bonsai_bf16_linear(_ptr(x), _ptr(w), _ptr(out), m, n, k, _stream(x.device))
     _need(rc == 0, f"bonsai_bf16_linear failed with status {rc}")
+    return out
+
+
+FP8_MAX = 448.0
+
+
+def prepare_fp8_weight(w: torch.Tensor):
+    """``(w_fp8 uint8 [ceil16(N), K], w_scale float)``: per-tensor scale ``amax|w| / 448`` and
+    E4M3 codes of ``w / w_scale`` with the rows padded to a multiple of 16 (reference:
+    ``prepare_fp8_lm_head``, model.py:1168-1194).  Done once at load time with torch's own cast."""
+    _need(w.dtype == torch.bfloat16 and w.dim() == 2, "w must be bf16 [N, K]")
+    n, k = w.shape
+    n_pad = -(-n // 16) * 16
+    wp = w
+    if n_pad != n:
+        wp = torch.zeros(n_pad, k, dtype=w.dtype, device=w.device)
+        wp[:n].copy_(w)
+    w_scale = (wp.abs().amax() / FP8_MAX).clamp_min(1e-12).to(torch.float32)
+    codes = (wp / w_scale).to(torch.float8_e4m3fn).view(torch.uint8).contiguous()
+    return codes, float(w_scale.item())
+
+
+def fp8_quant_rows(x: torch.Tensor, q: Optional[torch.Tensor] = None,
+                   scale: Optional[torch.Tensor] = None):
+    """Per-tensor E4M3 quantisation of a few bf16 rows: ``(q uint8 [M, K], scale fp32 [1])``
+    with ``scale = bf16(amax|x| / 448)`` and ``q = e4m3(bf16(x / scale))`` (reference:
+    model.py:1269-1270)."""
+    _check(x, torch.bfloat16, "x")
+    _need(x.dim() == 2 and 1 <= x.shape[0] <= MAX_WIDTH and x.shape[1] % 8 == 0,
+          f"x must be [1..{MAX_WIDTH}, K] with K a multiple of 8")
+    m, k = x.shape
+    if q is None:
+        q = torch.empty(m, k, dtype=torch.uint8, device=x.device)
+    if scale is None:
+        scale = torch.empty(1, dtype=torch.float32, device=x.device)
+    _check(q, torch.uint8, "q")
+    _check(scale, torch.float32, "scale")
+    _need(q.numel() >= m * k and scale.numel() >= 1, "fp8 output buffers too small")
+    with torch.cuda.device(x.device):
+        rc = decode_lib().bonsai_fp8_quant_rows(_ptr(x), _ptr(q), _ptr(scale), m, k, _stream(x.device))
+    _need(rc == 0, f"bonsai_fp8_quant_rows failed with status {rc}")
+    return q, scale
+
+
+def fp8_linear(x_q: torch.Tensor, x_scale: torch.Tensor, w_q: torch.Tensor, w_scale: float,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``bf16((x_q @ w_q.T) * x_scale * w_scale)`` for E4M3 codes ``x_q uint8 [M, K]`` and
+    ``w_q uint8 [N, K]`` (reference: ``torch._scaled_mm`` call of model.py:1271-1275)."""
+    _check(x_q, torch.uint8, "x_q")
+    _check(w_q, torch.uint8, "w_q")
+    _check(x_scale, torch.float32, "x_scale")
+    _need(x_q.dim() == 2 and w_q.dim() == 2 and x_q.shape[1] == w_q.shape[1], "x_q and w_q must share K")
+    m, k = x_q.shape
+    n = w_q.shape[0]
+    _need(1 <= m <= MAX_WIDTH and k % 128 == 0 and k >= 128, "fp8_linear: 1..32 rows, K a multiple of 128")
+    if out is None:
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=x_q.device)
+    else:
+        _check(out, torch.bfloat16, "out")
+        _need(out.numel() >= m * n, "out too small")
+    with torch.cuda.device(x_q.device):
+        rc = decode_lib().bonsai_fp8_linear(_ptr(x_q), _ptr(x_scale), _ptr(w_q), float(w_scale),
+                                            _ptr(out), m, n, k, _stream(x_q.device))
+    _need(rc == 0, f"bonsai_fp8_linear failed with status {rc}")
     return out

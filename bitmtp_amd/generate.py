@@ -30,6 +30,7 @@ from typing import Iterable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
+from . import contracts
 from .runtime import GraphAtlas
 
 
@@ -62,6 +63,26 @@ def verify_accept(draft_tokens: Sequence[int], verify_tokens: Sequence[int], D: 
             break
         n += 1
     return n
+
+
+def draft_role(atlas: GraphAtlas, use_fp8: bool, use_bf16: bool = False) -> str:
+    """The draft output-projection role: the exact native one, or one of the two
+    acceptance-tolerant approximations (``_draft_role``, fast_generate.py:586-599)."""
+    if use_fp8 and use_bf16:
+        raise RuntimeError("FP8 and BF16 draft roles are mutually exclusive")
+    role = "draft_fp8" if use_fp8 else ("draft_bf16" if use_bf16 else "draft")
+    if role not in atlas.roles:
+        raise RuntimeError(f"requested draft role was not captured: {role}")
+    return role
+
+
+def verify_role(atlas: GraphAtlas, use_fp8: bool = False, use_q1: bool = False,
+                use_w1a16: bool = False) -> str:
+    """Native verification only (``_verify_role``, fast_generate.py:602-608)."""
+    contracts.validate_native_verifier(use_fp8, use_q1, use_w1a16)
+    if "verify" not in atlas.roles:
+        raise RuntimeError("requested native verify role was not captured")
+    return "verify"
 
 
 def default_hybrid_m(D: int) -> int:
@@ -184,10 +205,19 @@ def _exact_m1_verify(atlas: GraphAtlas, sigma: int, cache_len: int, pending: Lis
 
 def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: float = 0.9,
                     hybrid_m: Optional[int] = None, max_gen_len: int = 512,
-                    eos_ids: Iterable[int] = (), exact_m1_verify: bool = False
+                    eos_ids: Iterable[int] = (), exact_m1_verify: bool = False,
+                    use_fp8_draft: bool = False, use_bf16_draft: bool = False,
+                    use_fp8_verify: bool = False, use_q1_verify: bool = False,
+                    use_w1a16_verify: bool = False, rabv_margin: float = 0.0
                     ) -> Tuple[List[int], dict]:
     """Hybrid decode: the confidence streak switches between draft-only commits and
-    verification (fast_generate.py:903-1187)."""
+    verification (fast_generate.py:903-1187).  Nonzero margins and non-native verifier
+    projections are rejected before anything touches the GPU (fast_generate.py:934-935);
+    ``use_fp8_draft`` / ``use_bf16_draft`` pick the approximate draft projection."""
+    contracts.validate_verification_options(rabv_margin, exact_m1_verify)
+    contracts.validate_native_verifier(use_fp8_verify, use_q1_verify, use_w1a16_verify)
+    role_d = draft_role(atlas, use_fp8_draft, use_bf16_draft)
+    role_v = verify_role(atlas)
     args = atlas.args
     D = args.block_size
     MASK = args.mask_token_id
@@ -238,7 +268,7 @@ def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: floa
                 sigma = new_sigma
 
         # ---- draft replay: [pending | pad | anchor | MASK x (D-1)]
-        gd = atlas.get_graph(M_draft, sigma, "draft")
+        gd = atlas.get_graph(M_draft, sigma, role_d)
         toks = pending + [0] * (P - n_pend) + [pending[-1]] + [MASK] * (D - 1)
         pos = [cache_len + i for i in range(n_pend)] + [0] * (P - n_pend) + \
               [cache_len + n_pend - 1 + i for i in range(D)]
@@ -259,7 +289,7 @@ def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: floa
                 accept_count, cache_len, bonus = _exact_m1_verify(
                     atlas, sigma, cache_len, pending, draft_tokens)
             else:
-                gv = atlas.get_graph(M_verify, sigma, "verify")
+                gv = atlas.get_graph(M_verify, sigma, role_v)
                 vt = [pending[-1]] + draft_tokens
                 vp = [cache_len - 1 + i for i in range(M_verify)]
                 atlas.replay(gv, vt, vp, cache_len)

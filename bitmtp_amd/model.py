@@ -225,11 +225,49 @@ class BonsaiDecoder:
             self.head_bf16 = None
             self.head_rows = head.out_features
 
+        self.head_fp8 = None        # (E4M3 codes uint8 [ceil16(vocab), dim], w_scale): draft_fp8
+        self.head_raw_bf16 = None   # bf16 [ceil8(vocab), dim]: draft_bf16
+
     @property
     def head_kind(self) -> str:
         if self.head is None:
             return "bf16"
         return "t2" if self.head.bits == 2 else "q1"
+
+    def _lm_head_weight(self) -> torch.Tensor:
+        """The bf16 output matrix ``[vocab, dim]``: the tied embedding (which a packed head
+        dequantises to) or the untied matrix (reference: model.py:1160-1166)."""
+        w = self.embed if self.head_bf16 is None else self.head_bf16
+        return w[: self.args.vocab_size]
+
+    def prepare_fp8_lm_head(self) -> None:
+        """E4M3 copy of the output matrix for the ``draft_fp8`` role (reference:
+        ``prepare_fp8_lm_head``, model.py:1168-1194)."""
+        if self.head_fp8 is None:
+            self.head_fp8 = decode_ops.prepare_fp8_weight(self._lm_head_weight())
+
+    def prepare_raw_bf16_head(self) -> None:
+        """The raw bf16 output matrix for the ``draft_bf16`` role (reference: precision
+        "bf16_raw", model.py:1276-1282), rows padded to a multiple of 8."""
+        if self.head_raw_bf16 is None:
+            if self.head_bf16 is not None:
+                self.head_raw_bf16 = self.head_bf16
+                return
+            w = self._lm_head_weight()
+            if w.shape[0] % 8:
+                padded = torch.zeros(-(-w.shape[0] // 8) * 8, w.shape[1], dtype=w.dtype, device=w.device)
+                padded[: w.shape[0]].copy_(w)
+                w = padded
+            self.head_raw_bf16 = w.contiguous()
+
+    def max_logits_ld(self) -> int:
+        """Largest leading dimension any prepared output projection writes."""
+        ld = self.head_rows
+        if self.head_fp8 is not None:
+            ld = max(ld, self.head_fp8[0].shape[0])
+        if self.head_raw_bf16 is not None:
+            ld = max(ld, self.head_raw_bf16.shape[0])
+        return ld
 
     # -- construction --------------------------------------------------------
     @classmethod
@@ -305,7 +343,8 @@ class Workspace:
     """Intermediate buffers of one step, sized for the widest graph and shared by all
     graphs (they replay one after another on one stream)."""
 
-    def __init__(self, args: ModelArgs, m_max: int, max_slots: int, head_rows: int, device):
+    def __init__(self, args: ModelArgs, m_max: int, max_slots: int, head_rows: int, device,
+                 logits_ld_max: int = 0):
         bf, i8, f32 = torch.bfloat16, torch.int8, torch.float32
 
         def buf(shape, dtype):
@@ -331,7 +370,15 @@ class Workspace:
         self.l_q = buf((m_max, args.dim), i8)
         self.l_s = buf((m_max,), f32)
         self.l_n = buf((m_max, args.dim), bf)
-        self.logits = buf((m_max, head_rows), bf)
+        self.l_f8 = buf((m_max, args.dim), torch.uint8)
+        self.l_f8_scale = buf((1,), f32)
+        # one buffer for the logits of every output projection; `logits` is its view with
+        # the native projection's leading dimension
+        self.logits_buf = buf((m_max * max(head_rows, logits_ld_max),), bf)
+        self.logits = self.logits_buf[: m_max * head_rows].view(m_max, head_rows)
+
+    def logits_view(self, rows: int, ld: int) -> torch.Tensor:
+        return self.logits_buf[: rows * ld].view(rows, ld)
 
 
 @dataclass
@@ -396,13 +443,15 @@ def _gemv(a_q: torch.Tensor, a_s: torch.Tensor, w: PackedLinear, out: torch.Tens
 
 def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tensor, sigma: int,
                  rope: Tuple[torch.Tensor, torch.Tensor], logits_start: int, logits_end: int,
-                 threshold: float) -> None:
+                 threshold: float, head_mode: str = "native") -> None:
     """Enqueue one width-``io.M`` step on the current stream.
 
     ``kv`` is the shared buffer ``[2, n_layers, n_kv, slots, 128]``; the new rows go to
     slots ``sigma .. sigma+M-1``.  Logit rows ``[logits_start, logits_end)`` are projected
     through the packed head; their argmax, confidence and accepted-prefix length land in
     ``io.tokens_out / io.conf / io.accept`` (rows counted from ``logits_start``).
+    ``head_mode``: "native" (the backbone's own projection), "fp8" or "bf16_raw" (the
+    approximate draft projections, model.py:1268-1282; prepared beforehand).
     """
     args = model.args
     M = io.M
@@ -448,20 +497,33 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
         _gemv(ws.i_q, ws.i_s, lw.w_down, ws.ffn_out, M, stream)
 
     rows = logits_end - logits_start
-    if model.head is None:
-        # bf16 projection of the normalised rows (reference: model.py:1401-1403 with
-        # lm_head_precision "bf16")
+    if head_mode not in ("native", "fp8", "bf16_raw"):
+        raise ValueError(f"unknown head_mode {head_mode!r}")
+    if head_mode != "native" or model.head is None:
+        # projections of the normalised bf16 rows (reference: model.py:1401-1403)
         check(actq.bonsai_add_rmsnorm_bf16(_vp(ws.ffn_out[logits_start:]), _vp(h_cur[logits_start:]),
                                            _vp(model.norm), eps, _vp(ws.h_last), _vp(ws.l_n),
                                            rows, dim, stream),
               "bonsai_add_rmsnorm_bf16")
-        decode_ops.bf16_linear(ws.l_n[:rows], model.head_bf16, ws.logits)
+        if head_mode == "fp8":
+            if model.head_fp8 is None:
+                raise RuntimeError("the FP8 draft projection was not prepared")
+            w_q, w_scale = model.head_fp8
+            logits = ws.logits_view(rows, w_q.shape[0])
+            decode_ops.fp8_quant_rows(ws.l_n[:rows], ws.l_f8, ws.l_f8_scale)
+            decode_ops.fp8_linear(ws.l_f8[:rows], ws.l_f8_scale, w_q, w_scale, logits)
+        else:
+            w = model.head_bf16 if head_mode == "native" else model.head_raw_bf16
+            if w is None:
+                raise RuntimeError("the raw bf16 draft projection was not prepared")
+            logits = ws.logits_view(rows, w.shape[0])
+            decode_ops.bf16_linear(ws.l_n[:rows], w, logits)
     else:
         check(actq.bonsai_add_rmsnorm_quant_int8(_vp(ws.ffn_out[logits_start:]),
                                                  _vp(h_cur[logits_start:]), _vp(model.norm), eps,
                                                  _vp(ws.h_last), _vp(ws.l_q), _vp(ws.l_s), rows,
                                                  dim, stream),
               "bonsai_add_rmsnorm_quant_int8")
-        _gemv(ws.l_q, ws.l_s, model.head, ws.logits, rows, stream)
-    decode_ops.draft_chain(ws.logits[:rows], args.vocab_size, threshold, io.tokens_out, io.conf,
-                           io.accept)
+        logits = ws.logits_view(rows, model.head_rows)
+        _gemv(ws.l_q, ws.l_s, model.head, logits, rows, stream)
+    decode_ops.draft_chain(logits, args.vocab_size, threshold, io.tokens_out, io.conf, io.accept)

@@ -19,13 +19,14 @@ Differences from the reference, by design:
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from . import decode_ops, ops
+from . import contracts, decode_ops, ops
 from .model import BonsaiDecoder, StepIO, Workspace, enqueue_step, rope_tables
 
 DEFAULT_SEGMENT_LADDER = (256, 1024, 4096)
@@ -64,10 +65,17 @@ def causal_row_masks(M: int) -> List[int]:
     return [(1 << (r + 1)) - 1 for r in range(M)]
 
 
+# output projection of each role: the backbone's own ("native"), the FP8 or the raw bf16
+# approximation for the acceptance-tolerant draft roles (fast_runtime.py:179-203)
+DRAFT_ROLES = ("draft", "draft_fp8", "draft_bf16")
+HEAD_MODE_OF_ROLE = {"ar": "native", "verify": "native", "draft": "native",
+                     "draft_fp8": "fp8", "draft_bf16": "bf16_raw"}
+
+
 def step_descriptor(role: str, M: int, D: int, cache_len: int, n_pend: int = 0) -> List[int]:
     """``[cache_len, hide, rowmask_0 .. rowmask_{M-1}]`` for one replay
     (reference: ``prepare_step`` / ``_prepare_verify``, fast_runtime.py:391-421,443-465)."""
-    if role == "draft":
+    if role in DRAFT_ROLES:  # the three draft roles share the mask
         P = M - D
         n_clamp = max(0, min(n_pend, P))
         hide = cache_len - 1 if (n_clamp == 0 and cache_len > 0) else -1
@@ -101,7 +109,7 @@ def logits_rows(role: str, M: int, D: int) -> Tuple[int, int]:
     """Rows projected through the head (reference: ``_capture_one``, fast_runtime.py:179-203)."""
     if role == "ar":
         return 0, M
-    if role == "draft":
+    if role in DRAFT_ROLES:
         return M - D, M
     if role == "verify":
         return 0, min(D + 1, M)
@@ -131,9 +139,7 @@ class GraphAtlas:
                  threshold: float = 0.9,
                  prefill_width: int = 16,
                  use_graphs: bool = True):
-        for r in roles:
-            if r not in ROLES:
-                raise ValueError(f"unsupported graph role: {r!r}")
+        contracts.validate_graph_roles(roles)
         self.model = model
         self.args = model.args
         self.device = model.device
@@ -150,7 +156,15 @@ class GraphAtlas:
         ops.init_kernels()
         self.kv_buffers: Dict[int, torch.Tensor] = {}
         max_slots = self.segment_ladder[-1] + self.M_max
-        self.workspace = Workspace(self.args, self.M_max, max_slots, model.head_rows, self.device)
+        # the approximate draft projections are prepared once, like the reference does in
+        # GraphAtlas.__init__ (fast_runtime.py:112-118)
+        if "draft_fp8" in self.roles:
+            contracts.validate_graph_roles(self.roles, torch.cuda.get_device_capability(self.device))
+            model.prepare_fp8_lm_head()
+        if "draft_bf16" in self.roles:
+            model.prepare_raw_bf16_head()
+        self.workspace = Workspace(self.args, self.M_max, max_slots, model.head_rows, self.device,
+                                   logits_ld_max=model.max_logits_ld())
         self.rope = rope_tables(self.args, max_slots, self.device)
         self.graphs: Dict[Tuple[int, int, str], CapturedGraph] = {}
         self.replays = 0
@@ -210,20 +224,33 @@ class GraphAtlas:
                         self.get_graph(1, sigma, "ar")
                     continue
                 for role in self.roles:
-                    if role == "ar" or (role == "draft" and M < self.D) or \
+                    if role == "ar" or (role in DRAFT_ROLES and M < self.D) or \
                             (role == "verify" and M != self.D + 1):
                         continue
                     self.get_graph(M, sigma, role)
 
     def _capture_one(self, M: int, sigma: int, role: str) -> CapturedGraph:
-        # capture keeps process-wide state tensors; they must not become inference tensors
-        with torch.inference_mode(False):
-            return self._capture_one_impl(M, sigma, role)
+        # The cyclic garbage collector must not run while a stream is capturing: if it finds
+        # an unreachable atlas, it destroys that atlas's graphs in the middle of this capture,
+        # which aborts the process.  Collect first, then keep the collector off until the
+        # capture has ended.  (Capture keeps process-wide state tensors; they must not become
+        # inference tensors, hence inference_mode(False).)
+        gc.collect()
+        gc_was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.inference_mode(False):
+                return self._capture_one_impl(M, sigma, role)
+        finally:
+            if gc_was_enabled:
+                gc.enable()
 
     def _capture_one_impl(self, M: int, sigma: int, role: str) -> CapturedGraph:
-        if role not in ROLES:
+        if role not in contracts.GRAPH_ROLES:
             raise ValueError(f"unsupported graph role: {role!r}")
-        if role == "draft" and M < self.D:
+        if role not in self.roles:
+            raise RuntimeError(f"graph role {role!r} was not requested for this atlas")
+        if role in DRAFT_ROLES and M < self.D:
             raise ValueError(f"a draft graph needs M >= D = {self.D}")
         if M > self.M_max:
             raise ValueError(f"width {M} exceeds the atlas maximum {self.M_max}")
@@ -235,9 +262,13 @@ class GraphAtlas:
         io.step_in_host[: 2 + M] = torch.tensor(desc, dtype=torch.int32)
         io.step_in.copy_(io.step_in_host)
 
+        # the closure holds the pieces, not the atlas: no reference cycle through the graphs
+        model, workspace, rope, threshold = self.model, self.workspace, self.rope, self.threshold
+        head_mode = HEAD_MODE_OF_ROLE[role]
+
         def run():
-            enqueue_step(self.model, self.workspace, io, kv, sigma, self.rope, ls, le,
-                         self.threshold)
+            enqueue_step(model, workspace, io, kv, sigma, rope, ls, le, threshold,
+                         head_mode=head_mode)
 
         graph = None
         if self.use_graphs:

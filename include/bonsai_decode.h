@@ -113,6 +113,24 @@ int bonsai_draft_chain(const void *logits, int rows, int ld, int vocab, float th
  * a function attribute: make it outside stream capture. */
 int bonsai_bf16_linear(const void *x, const void *w, void *out, int M, int N, int K, void *stream);
 
+/* FP8 draft projection (the acceptance-tolerant `draft_fp8` role): the run-time half of
+ * `_lm_head` with precision "fp8" (src/bonsai_sft/gpu/model.py:1268-1275).
+ *   h_scale = fp32( max( bf16(amax(|x|) / 448), bf16(1e-12) ) )   one scale for all M rows,
+ *                                                     evaluated in bf16 like the tensor expression
+ *   q       = e4m3fn( bf16( fp32(x) / h_scale ) )       OCP E4M3, round to nearest even
+ * x bf16 [M, K] (M <= BONSAI_MAX_WIDTH, K % 8 == 0), q uint8 [M, K], scale fp32 [1] (device). */
+int bonsai_fp8_quant_rows(const void *x, void *q, float *scale, int M, int K, void *stream);
+
+/* out = bf16( (x_fp8 @ w_fp8^T) * x_scale[0] * w_scale ): `torch._scaled_mm(h_fp8, W.T,
+ * scale_a, scale_b, out_dtype=bf16)` of model.py:1271-1275, with the weight matrix
+ * prepared as in `prepare_fp8_lm_head` (model.py:1168-1194: w_scale = amax(|W|)/448,
+ * W_fp8 = e4m3fn(W / w_scale), rows padded to a multiple of 16).
+ *   x uint8 [M, K] E4M3, x_scale fp32 [1] (device), w uint8 [N, K] E4M3, out bf16 [M, N];
+ *   K % 128 == 0.  fp32 accumulation in a fixed order; compared with a float64 product of the
+ * same FP8 operands to one bf16 step.  First call per device outside stream capture. */
+int bonsai_fp8_linear(const void *x, const float *x_scale, const void *w, float w_scale, void *out,
+                      int M, int N, int K, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -175,6 +175,18 @@ def test_draft_chain_kernel(DO, rows, vocab, ld):
 
 
 # ---------------------------------------------------------------- bf16 output projection
+def _assert_one_bf16_step(got: torch.Tensor, want64: torch.Tensor) -> None:
+    """fp32 accumulation against a float64 product: the same or the adjacent bf16 value
+    wherever the result is not a cancellation (>= 2 % of the largest), a small absolute
+    error elsewhere (there the fp32 summation order shows in the last places)."""
+    want_b = want64.to(torch.bfloat16)
+    d = np.abs(bf16_ordinal(bf16_bits(got)) - bf16_ordinal(bf16_bits(want_b)))
+    top = want64.abs().max().item()
+    big = (want64.abs() >= 0.02 * top).cpu().numpy()
+    assert d[big].max() <= 1 and (d[big] != 0).mean() < 0.05
+    assert (got.double() - want64).abs().max().item() <= 2.0 ** -8 * top
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1000, 512), (9, 4099, 2048), (16, 1536, 2560), (17, 300, 64),
                                    (32, 129, 128), (3, 7, 320), (5, 151936, 2048)])
 def test_bf16_linear_against_fp32_matmul(M, N, K):
@@ -187,16 +199,58 @@ def test_bf16_linear_against_fp32_matmul(M, N, K):
     print(f"[case] bf16_linear M={M} N={N} K={K}", flush=True)
     got = decode_ops.bf16_linear(x, w)
     torch.cuda.synchronize()
-    want = (x.double() @ w.double().T)
-    want_b = want.to(torch.bfloat16)
-    d = np.abs(bf16_ordinal(bf16_bits(got)) - bf16_ordinal(bf16_bits(want_b)))
-    small = (want.abs() < 1e-3 * want.abs().max()).cpu().numpy()
-    assert d[~small].max() <= 1
-    assert (d[~small] != 0).mean() < 0.05
-    assert (got.double() - want).abs().max().item() <= 1e-2 * want.abs().max().item()
+    _assert_one_bf16_step(got, x.double() @ w.double().T)
     # a preallocated output with a wider leading dimension is rejected, wrong K as well
     with pytest.raises(RuntimeError):
         decode_ops.bf16_linear(x, w[:, : K - 64].contiguous() if K > 64 else w[:, :32].contiguous())
+
+
+# ---------------------------------------------------------------- FP8 draft projection
+@pytest.mark.parametrize("M,K", [(1, 128), (8, 2048), (17, 2560), (3, 264)])
+def test_fp8_row_quantiser_matches_torch_cast(M, K):
+    """scale and codes are the reference's tensor expression (model.py:1269-1270) evaluated
+    by this build's own PyTorch on the CPU, bit for bit."""
+    from bitmtp_amd import decode_ops
+    rng = np.random.default_rng(M + K)
+    x = _rand_bf16(rng, (M, K), 3.0)
+    x[0, :8] = torch.tensor([0.0, -0.0, 1e-4, -1e-4, 2e-3, 7.0, -7.0, 0.013], dtype=torch.bfloat16)
+    print(f"[case] fp8_quant_rows M={M} K={K}", flush=True)
+    q, s = decode_ops.fp8_quant_rows(x.to(DEV))
+    torch.cuda.synchronize()
+    h_scale = (x.abs().amax() / 448.0).clamp_min(1e-12).to(torch.float32)
+    want = (x / h_scale).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert s.cpu().item() == h_scale.item()
+    got = q.cpu()
+    # -0 and +0 results are the same value; everything else is the same code
+    same = (got == want) | (((got | want) & 0x7F) == 0)
+    assert bool(same.all())
+    # an all-zero tensor takes the clamp: scale bf16(1e-12), codes zero
+    q0, s0 = decode_ops.fp8_quant_rows(torch.zeros(2, 128, dtype=torch.bfloat16, device=DEV))
+    assert s0.cpu().item() == torch.tensor(1e-12).to(torch.bfloat16).float().item()
+    assert int(q0.cpu().max()) == 0
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1008, 512), (8, 4112, 2048), (16, 1536, 2560), (17, 304, 128),
+                                   (9, 151936, 2048)])
+def test_fp8_linear_against_float64_product(M, N, K):
+    from bitmtp_amd import decode_ops
+    rng = np.random.default_rng(M * 7 + N + K)
+    w = _rand_bf16(rng, (N - 5, K), 0.03).to(DEV)
+    x = _rand_bf16(rng, (M, K), 2.0).to(DEV)
+    w_q, w_scale = decode_ops.prepare_fp8_weight(w)
+    assert tuple(w_q.shape) == (N, K) and w_q.dtype == torch.uint8      # rows padded to 16
+    assert bool((w_q[N - 5:] == 0).all())
+    x_q, x_scale = decode_ops.fp8_quant_rows(x)
+    print(f"[case] fp8_linear M={M} N={N} K={K}", flush=True)
+    got = decode_ops.fp8_linear(x_q, x_scale, w_q, w_scale)
+    torch.cuda.synchronize()
+    xf = x_q.view(torch.float8_e4m3fn).double()
+    wf = w_q.view(torch.float8_e4m3fn).double()
+    want = (xf @ wf.T) * float(x_scale.item()) * w_scale
+    _assert_one_bf16_step(got, want)
+    # and the FP8 projection approximates the bf16 one it stands in for
+    exact = x.double() @ torch.cat([w, torch.zeros(5, K, dtype=w.dtype, device=DEV)]).double().T
+    assert (got.double() - exact).abs().max().item() <= 0.08 * exact.abs().max().item()
 
 
 # ---------------------------------------------------------------- whole step and loops
@@ -480,3 +534,51 @@ def test_decoder_rejects_mixed_weight_kinds():
         BonsaiDecoder(_tiny_args(kernel_kind="q1"), model.layers, model.embed, model.norm, None)
     with pytest.raises(ValueError):
         BonsaiDecoder.random_init(_tiny_args(kernel_kind="w4"), seed=3, device=DEV)
+
+
+# ---------------------------------------------------------------- approximate draft roles
+@pytest.mark.parametrize("kind", ["t2g128", "q1"])
+def test_fp8_and_bf16_draft_roles(kind):
+    """The acceptance-tolerant draft projections (fast_runtime.py:188-199): their logits stay
+    close to the native ones, verification stays native, so hybrid decode with exact width-1
+    verification still reproduces AR token for token, and a role that was not requested for
+    the atlas is refused."""
+    from bitmtp_amd import generate
+    from bitmtp_amd.model import BonsaiDecoder
+    from bitmtp_amd.runtime import GraphAtlas
+    model = BonsaiDecoder.random_init(_tiny_args(kernel_kind=kind), seed=17, device=DEV)
+    atlas = GraphAtlas(model, segment_ladder=(64, 256), threshold=0.9,
+                       roles=("ar", "draft", "draft_fp8", "draft_bf16", "verify"))
+    assert model.head_fp8[0].shape == (1008, 512) and model.head_raw_bf16.shape == (1000, 512)
+    rng = np.random.default_rng(31)
+    sigma, cache_len, M = 64, 19, 9
+    hist = _rand_bf16(rng, tuple(atlas.kv(sigma).shape), 0.5).to(DEV)
+    tokens = rng.integers(0, 1000, M).tolist()
+    positions = [cache_len + i for i in range(M)]
+    logits = {}
+    for role in ("draft", "draft_fp8", "draft_bf16"):
+        atlas.kv(sigma).copy_(hist)
+        g = atlas.get_graph(M, sigma, role)
+        print(f"[case] {kind} role {role}", flush=True)
+        for _ in range(2):   # a replay after the first gives the same result
+            atlas.replay(g, tokens, positions, cache_len, n_pend=1)
+            toks, conf, accept = atlas.read_outputs(g)
+            rows = g.logits_end - g.logits_start
+            ld = {"draft": model.head_rows, "draft_fp8": 1008, "draft_bf16": 1000}[role]
+            cur = atlas.workspace.logits_view(rows, ld)[:, :1000].float().cpu().numpy()
+            if role in logits:
+                assert np.array_equal(cur, logits[role])
+            logits[role] = cur
+            assert toks.tolist() == cur.argmax(-1).tolist()
+    ref = logits["draft"]
+    scale = np.abs(ref).max()
+    assert np.abs(logits["draft_bf16"] - ref).max() <= 0.05 * scale
+    assert np.abs(logits["draft_fp8"] - ref).max() <= 0.12 * scale
+    prompt = rng.integers(0, 1000, 21).tolist()
+    ar, _ = generate.ar_generate(atlas, prompt, max_gen_len=24)
+    for kw in ({"use_fp8_draft": True}, {"use_bf16_draft": True}):
+        hy, st = generate.hybrid_generate(atlas, prompt, max_gen_len=24, exact_m1_verify=True, **kw)
+        assert hy == ar
+    plain = GraphAtlas(model, segment_ladder=(64,))
+    with pytest.raises(RuntimeError, match="not captured"):
+        generate.hybrid_generate(plain, prompt, max_gen_len=4, use_fp8_draft=True)

@@ -100,7 +100,9 @@ def test_draft_template_rows_follow_the_specification():
 
 def test_unknown_role_and_bad_pending_are_rejected():
     with pytest.raises(ValueError, match="unsupported graph role"):
-        R.step_descriptor("draft_fp8", 9, 8, 3, 1)
+        R.step_descriptor("verify_q1", 9, 8, 3, 1)
+    with pytest.raises(ValueError, match="unsupported graph role"):
+        R.logits_rows("draft_int4", 9, 8)
     with pytest.raises(ValueError):
         R.draft_row_masks(9, 8, 2)
     assert R.logits_rows("ar", 1, 8) == (0, 1)
@@ -132,6 +134,55 @@ def test_verify_accept_known_answers():
     assert G.verify_accept([1, 0], verifier, 2) == 0
     assert G.verify_accept([0, 1], verifier, 2) == 1
     assert G.verify_accept([0, 0], verifier, 2) == 2
+
+
+def test_margins_and_foreign_verifiers_are_rejected_before_gpu_use():
+    """tests/test_bonsai_strict_verifier.py:38-52 of the reference: every nonzero margin and
+    every non-native verifier flag raises before the atlas is touched."""
+    from bitmtp_amd import contracts
+    for margin in (-0.5, 1e-20, 0.5, float("inf"), float("nan")):
+        with pytest.raises(ValueError, match="requires rabv_margin=0"):
+            G.hybrid_generate(None, None, rabv_margin=margin)
+    for flag in ("use_fp8_verify", "use_q1_verify", "use_w1a16_verify"):
+        with pytest.raises(ValueError, match="native verifier projection"):
+            G.hybrid_generate(None, None, **{flag: True})
+    contracts.validate_verification_options(0.0)
+    contracts.validate_verification_options(-0.0, exact_m1_verify=True)
+    with pytest.raises(ValueError):
+        contracts.validate_verification_options("0.1")
+
+
+def test_draft_and_verifier_role_selection():
+    """tests/test_bonsai_strict_verifier.py:54-68 and :103-110 of the reference."""
+    from bitmtp_amd import contracts
+    atlas = SimpleNamespace(roles=("draft", "draft_fp8", "draft_bf16", "verify"))
+    assert G.draft_role(atlas, False) == "draft"
+    assert G.draft_role(atlas, False, True) == "draft_bf16"
+    assert G.draft_role(atlas, True) == "draft_fp8"
+    assert G.verify_role(atlas, False) == "verify"
+    with pytest.raises(ValueError, match="native verifier"):
+        G.verify_role(atlas, False, True)
+    with pytest.raises(RuntimeError, match="mutually exclusive"):
+        G.draft_role(atlas, True, True)
+    with pytest.raises(ValueError, match="native verifier"):
+        G.verify_role(atlas, True, True)
+    with pytest.raises(RuntimeError, match="not captured"):
+        G.draft_role(SimpleNamespace(roles=("draft", "verify")), True)
+    with pytest.raises(RuntimeError, match="not captured"):
+        G.verify_role(SimpleNamespace(roles=("draft",)))
+    contracts.validate_graph_roles(("ar", "draft_bf16", "verify"), (8, 6))
+    contracts.validate_graph_roles(("ar", "draft", "verify"), (8, 6))
+    contracts.validate_graph_roles(("ar", "draft_fp8", "verify"), (9, 5))
+    with pytest.raises(ValueError, match="FP8 draft"):
+        contracts.validate_graph_roles(("ar", "draft_fp8", "verify"), (8, 6))
+    with pytest.raises(ValueError, match="unsupported strict graph roles"):
+        contracts.validate_graph_roles(("ar", "verify_q1"))
+    # the approximate draft roles share the draft mask and logit rows
+    for role in ("draft_fp8", "draft_bf16"):
+        assert R.step_descriptor(role, 12, 8, 30, 3) == R.step_descriptor("draft", 12, 8, 30, 3)
+        assert R.logits_rows(role, 12, 8) == (4, 12)
+        assert R.HEAD_MODE_OF_ROLE[role] in ("fp8", "bf16_raw")
+    assert {R.HEAD_MODE_OF_ROLE[r] for r in ("ar", "draft", "verify")} == {"native"}
 
 
 def test_draft_chain_known_answer():
