@@ -216,6 +216,8 @@ def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: floa
     ``use_fp8_draft`` / ``use_bf16_draft`` pick the approximate draft projection."""
     contracts.validate_verification_options(rabv_margin, exact_m1_verify)
     contracts.validate_native_verifier(use_fp8_verify, use_q1_verify, use_w1a16_verify)
+    if hybrid_m is not None and hybrid_m < 1:
+        raise ValueError("hybrid_m must be at least 1")
     role_d = draft_role(atlas, use_fp8_draft, use_bf16_draft)
     role_v = verify_role(atlas)
     args = atlas.args
@@ -360,4 +362,26 @@ def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: floa
         "conf_path_frac": n_conf_path / max(1, n_conf_path + n_verify_path),
         "n_conf_path": n_conf_path, "n_verify_path": n_verify_path,
     })
+    return gen, st
+
+
+def speculative_generate(atlas: GraphAtlas, input_ids: Sequence[int], max_gen_len: int = 512,
+                         eos_ids: Iterable[int] = (), exact_m1_verify: bool = False,
+                         use_fp8_draft: bool = False, use_bf16_draft: bool = False,
+                         use_fp8_verify: bool = False, use_q1_verify: bool = False,
+                         use_w1a16_verify: bool = False, rabv_margin: float = 0.0
+                         ) -> Tuple[List[int], dict]:
+    """Self-speculative decode (fast_generate.py:664-899): every iteration drafts D tokens,
+    verifies them with the width-(D+1) graph (or the exact width-1 path) and commits the
+    matching prefix plus the verifier's bonus token.  It is the hybrid loop with the
+    confidence path switched off: a chain length never reaches D + 1."""
+    gen, st = hybrid_generate(atlas, input_ids, threshold=float("inf"),
+                              hybrid_m=atlas.args.block_size + 1 if atlas is not None else None,
+                              max_gen_len=max_gen_len, eos_ids=eos_ids,
+                              exact_m1_verify=exact_m1_verify, use_fp8_draft=use_fp8_draft,
+                              use_bf16_draft=use_bf16_draft, use_fp8_verify=use_fp8_verify,
+                              use_q1_verify=use_q1_verify, use_w1a16_verify=use_w1a16_verify,
+                              rabv_margin=rabv_margin)
+    if st["n_conf_path"] != 0:
+        raise RuntimeError("speculative decode took a confidence path")
     return gen, st

@@ -387,6 +387,25 @@ def test_hybrid_with_exact_verification_reproduces_ar(tiny):
     assert st["decode_tokens"] == 1 + st["accepted_drafts"] + st["verifier_bonus_tokens"]
 
 
+def test_speculative_decode_always_verifies(tiny):
+    """fast_generate.py:664-899: draft + verify every iteration; with the exact width-1
+    verifier the tokens are the AR ones, with the width-(D+1) verifier every committed
+    token is a verifier-approved draft or a verifier bonus."""
+    from bitmtp_amd import generate
+    model, atlas = tiny
+    rng = np.random.default_rng(29)
+    prompt = rng.integers(0, 1000, 23).tolist()
+    ar, _ = generate.ar_generate(atlas, prompt, max_gen_len=30)
+    sp, st = generate.speculative_generate(atlas, prompt, max_gen_len=30, exact_m1_verify=True)
+    assert sp == ar
+    assert st["n_conf_path"] == 0 and st["conf_path_frac"] == 0.0
+    assert st["n_verify_path"] == st["draft_iters"] and st["drafted_tokens"] == 8 * st["draft_iters"]
+    sp2, st2 = generate.speculative_generate(atlas, prompt, max_gen_len=30)
+    assert len(sp2) == 30 and st2["n_conf_path"] == 0
+    assert st2["decode_tokens"] == 1 + st2["accepted_drafts"] + st2["verifier_bonus_tokens"]
+    assert sp2[0] == ar[0]
+
+
 @pytest.mark.parametrize("threshold,hybrid_m", [(0.9, None), (0.0, 1), (0.0, 8)])
 def test_hybrid_accounting_and_width_schedule(tiny, threshold, hybrid_m):
     from bitmtp_amd import generate

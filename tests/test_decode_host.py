@@ -140,12 +140,13 @@ def test_margins_and_foreign_verifiers_are_rejected_before_gpu_use():
     """tests/test_bonsai_strict_verifier.py:38-52 of the reference: every nonzero margin and
     every non-native verifier flag raises before the atlas is touched."""
     from bitmtp_amd import contracts
-    for margin in (-0.5, 1e-20, 0.5, float("inf"), float("nan")):
-        with pytest.raises(ValueError, match="requires rabv_margin=0"):
-            G.hybrid_generate(None, None, rabv_margin=margin)
-    for flag in ("use_fp8_verify", "use_q1_verify", "use_w1a16_verify"):
-        with pytest.raises(ValueError, match="native verifier projection"):
-            G.hybrid_generate(None, None, **{flag: True})
+    for generate in (G.speculative_generate, G.hybrid_generate):
+        for margin in (-0.5, 1e-20, 0.5, float("inf"), float("nan")):
+            with pytest.raises(ValueError, match="requires rabv_margin=0"):
+                generate(None, None, rabv_margin=margin)
+        for flag in ("use_fp8_verify", "use_q1_verify", "use_w1a16_verify"):
+            with pytest.raises(ValueError, match="native verifier projection"):
+                generate(None, None, **{flag: True})
     contracts.validate_verification_options(0.0)
     contracts.validate_verification_options(-0.0, exact_m1_verify=True)
     with pytest.raises(ValueError):
