@@ -385,3 +385,102 @@ def speculative_generate(atlas: GraphAtlas, input_ids: Sequence[int], max_gen_le
     if st["n_conf_path"] != 0:
         raise RuntimeError("speculative decode took a confidence path")
     return gen, st
+
+
+def confidence_accept(tokens: Sequence[int], conf: Sequence[float], threshold: float, eos_set,
+                      D: int) -> Tuple[List[int], int, bool]:
+    """Confidence-streak acceptance of one block (``_confidence_accept``,
+    fast_generate.py:354-386): ``1 + longest streak of conf[1:] > threshold`` tokens, cut in
+    front of the first EOS among them; returns ``(accepted, count, eos_hit)``."""
+    n = min(draft_chain_accept(conf[:D], threshold), D)
+    accepted: List[int] = []
+    for t in tokens[:n]:
+        if int(t) in eos_set:
+            return accepted, len(accepted), True
+        accepted.append(int(t))
+    return accepted, n, False
+
+
+def confidence_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: float = 0.9,
+                        max_gen_len: int = 512, eos_ids: Iterable[int] = (),
+                        use_fp8_draft: bool = False, use_bf16_draft: bool = False
+                        ) -> Tuple[List[int], dict]:
+    """Confidence-chain decode (fast_generate.py:393-572): every iteration commits the
+    confident prefix of a drafted block and re-forwards it as pending rows of the next; no
+    verifier.  The first block is drafted straight after the prompt from the last prompt
+    token as anchor (positions seq_len-1 .. seq_len+D-2, its history copy hidden), which the
+    reference runs as a variable-shape forward (fast_generate.py:322-352) and this harness as
+    the width-D draft graph with no pending rows: the same mask
+    (``create_sdlm_attention_mask``, model.py:462-505)."""
+    role = draft_role(atlas, use_fp8_draft, use_bf16_draft)
+    args = atlas.args
+    D, MASK, dev = args.block_size, args.mask_token_id, atlas.device
+    eos_set = set(int(e) for e in eos_ids)
+    prompt = [int(t) for t in input_ids]
+    seq_len = len(prompt)
+
+    t0 = time.time()
+    sigma = atlas.select_segment(seq_len + max_gen_len + atlas.M_max)
+    prefill(atlas, prompt, sigma)
+    cache_len = seq_len
+    g1 = atlas.get_graph(D, sigma, role)
+    atlas.replay(g1, [prompt[-1]] + [MASK] * (D - 1),
+                 [seq_len - 1 + i for i in range(D)], cache_len, n_pend=0)
+    toks, conf, _ = atlas.read_outputs(g1)
+    accepted, _, eos_found = confidence_accept(toks, conf, threshold, eos_set, D)
+    torch.cuda.synchronize(dev)
+    prefill_time = time.time() - t0
+
+    gen: List[int] = list(accepted[:max_gen_len])
+    untimed = len(gen)
+    n_iters = 1
+    accept_total = len(gen)
+    pending = list(gen)
+    t1 = time.time()
+    while len(gen) < max_gen_len and not eos_found and pending:
+        n_iters += 1
+        n_pend = len(pending)
+        M = select_M_for_pending(atlas, n_pend)
+        P = M - D
+        if n_pend > P:
+            raise RuntimeError(f"{n_pend} pending tokens do not fit the widest draft graph")
+        if cache_len + atlas.M_max > sigma:
+            new_sigma = atlas.select_segment(cache_len + atlas.M_max + 64)
+            if new_sigma != sigma:
+                atlas.migrate_segment(sigma, new_sigma, cache_len)
+                sigma = new_sigma
+        g = atlas.get_graph(M, sigma, role)
+        toks_in = pending + [0] * (P - n_pend) + [pending[-1]] + [MASK] * (D - 1)
+        pos = [cache_len + i for i in range(n_pend)] + [0] * (P - n_pend) + \
+              [cache_len + n_pend - 1 + i for i in range(D)]
+        atlas.replay(g, toks_in, pos, cache_len, n_pend=n_pend)
+        atlas.commit_kv(sigma, cache_len, n_pend)
+        cache_len += n_pend
+        toks, conf, _ = atlas.read_outputs(g)
+        accepted, n_acc, eos_hit = confidence_accept(toks, conf, threshold, eos_set, D)
+        remaining = max(0, max_gen_len - len(gen))
+        if n_acc > remaining:
+            accepted = accepted[:remaining]
+            n_acc = len(accepted)
+        accept_total += n_acc
+        pending = accepted
+        if n_acc == 0:
+            break
+        gen.extend(accepted)
+        eos_found = eos_hit
+        if cache_len + n_pend + D > atlas.segment_ladder[-1]:
+            break
+    torch.cuda.synchronize(dev)
+    decode_time = max(time.time() - t1, 1e-9)
+    n_out = len(gen)
+    st = {
+        "prefill_time": prefill_time, "decode_time": decode_time if n_iters > 1 else 1e-9,
+        "total_time": time.time() - t0, "prefill_tokens": seq_len, "decode_tokens": n_out,
+        "timed_decode_tokens": max(0, n_out - untimed), "untimed_output_tokens": untimed,
+        "n_iters": n_iters, "avg_accept": accept_total / max(1, n_iters), "ttft": prefill_time,
+        "draft_iters": n_iters, "drafted_tokens": D * n_iters, "accepted_drafts": n_out,
+        "accept_rate": n_out / max(1, D * n_iters), "verifier_bonus_tokens": 0,
+        "committed_tokens": n_out, "committed_per_iter": n_out / max(1, n_iters),
+        "conf_path_frac": 1.0, "n_conf_path": n_iters, "n_verify_path": 0,
+    }
+    return gen, st

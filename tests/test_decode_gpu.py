@@ -406,6 +406,31 @@ def test_speculative_decode_always_verifies(tiny):
     assert sp2[0] == ar[0]
 
 
+def test_confidence_decode(tiny):
+    """fast_generate.py:393-572: blocks are committed on confidence alone.  Threshold 0
+    commits whole blocks, an infinite threshold one token per iteration; the first block is
+    drafted from the last prompt token, so its first token is the AR one."""
+    from bitmtp_amd import generate
+    model, atlas = tiny
+    rng = np.random.default_rng(41)
+    prompt = rng.integers(0, 1000, 27).tolist()
+    ar, _ = generate.ar_generate(atlas, prompt, max_gen_len=4)
+    full, st = generate.confidence_generate(atlas, prompt, threshold=0.0, max_gen_len=50)
+    assert len(full) == 50 and full[0] == ar[0]
+    assert st["n_iters"] == 7 and st["untimed_output_tokens"] == 8       # 6 x 8 + 2
+    assert st["timed_decode_tokens"] == 42 and st["n_verify_path"] == 0 and st["conf_path_frac"] == 1.0
+    assert st["drafted_tokens"] == 8 * st["n_iters"] and st["accepted_drafts"] == 50
+    again, _ = generate.confidence_generate(atlas, prompt, threshold=0.0, max_gen_len=50)
+    assert again == full
+    one, st1 = generate.confidence_generate(atlas, prompt, threshold=float("inf"), max_gen_len=12)
+    assert len(one) == 12 and st1["n_iters"] == 12 and st1["untimed_output_tokens"] == 1
+    assert one[0] == full[0]
+    # an EOS inside the first block ends the run in front of it
+    cut, stc = generate.confidence_generate(atlas, prompt, threshold=0.0, max_gen_len=50,
+                                            eos_ids=[full[3]])
+    assert cut == full[:full.index(full[3])] and stc["n_iters"] == 1
+
+
 @pytest.mark.parametrize("threshold,hybrid_m", [(0.9, None), (0.0, 1), (0.0, 8)])
 def test_hybrid_accounting_and_width_schedule(tiny, threshold, hybrid_m):
     from bitmtp_amd import generate

@@ -186,6 +186,21 @@ def test_draft_and_verifier_role_selection():
     assert {R.HEAD_MODE_OF_ROLE[r] for r in ("ar", "draft", "verify")} == {"native"}
 
 
+def test_confidence_accept_known_answers():
+    """``_confidence_accept`` (fast_generate.py:354-386): streak after the first token, cut in
+    front of an EOS, at least the anchor's prediction."""
+    toks = [5, 6, 7, 8, 9, 10, 11, 12]
+    conf = [0.1, 0.95, 0.97, 0.5, 0.99, 0.99, 0.99, 0.99]
+    assert G.confidence_accept(toks, conf, 0.9, set(), 8) == ([5, 6, 7], 3, False)
+    assert G.confidence_accept(toks, [0.0] + [1.0] * 7, 0.9, set(), 8) == (toks, 8, False)
+    assert G.confidence_accept(toks, [1.0] + [0.0] * 7, 0.9, set(), 8) == ([5], 1, False)
+    assert G.confidence_accept(toks, conf, 0.9, {6}, 8) == ([5], 1, True)
+    assert G.confidence_accept(toks, conf, 0.9, {5}, 8) == ([], 0, True)
+    assert G.confidence_accept(toks, conf, 0.9, {8}, 8) == ([5, 6, 7], 3, False)   # beyond the streak
+    # NaN never passes the gate
+    assert G.confidence_accept(toks, [0.5, float("nan"), 1.0], 0.9, set(), 8)[1] == 1
+
+
 def test_draft_chain_known_answer():
     logits = np.array([[0., 0.], [20., 0.], [0., 0.], [20., 0.]], dtype=np.float32)
     tokens, conf, length = DO.draft_chain(logits, 0.9)
