@@ -254,6 +254,275 @@ attn_partial_kernel(const uint32_t *pq, const uint32_t *pk, const uint32_t *pv, 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Matrix-core form of the chunk pass.  The VALU form above gives every (query head, row
+// group) its own wave, so a chunk of K/V is fetched from L2 by heads-per-group x row-groups
+// waves, each lane loading its own 256-byte row; from a few hundred slots on that L2
+// traffic is what the launch waits for.  Here a workgroup of four waves takes a tile of up
+// to 16 (row, query head) pairs of one kv head -- all query heads of the group and as many
+// block rows as fit -- and a run of consecutive 64-slot chunks.  Wave w owns slots
+// 16 w .. 16 w + 15 of the chunk for the scores and dims 32 w .. 32 w + 31 of the output:
+//   S = Q K^T      4 x v_mfma_f32_16x16x32_bf16 per wave: A = the pair tile's q rows, B = K
+//                  rows loaded straight in operand layout (lane = (slot, 8 dims of a 32-dim
+//                  block): four lanes cover 64 contiguous bytes of a K row);
+//   softmax        running max / sum per pair in base 2: the D layout keeps a pair's 16
+//                  scores of the wave in one 16-lane row (DPP row reductions), the four
+//                  waves exchange their maxima and sums through LDS; p is rounded to bf16
+//                  as the reference's probabilities are (model.py:1001) and the sum is
+//                  taken over the rounded values;
+//   O += P V       4 more MFMAs per wave: V rows are fetched coalesced, staged in LDS (row
+//                  pitch 288 bytes: conflict-free) and read back as 8 slots x 1 dim per
+//                  lane; P goes through LDS into A-operand order.  The slot <-> (K-block,
+//                  element) assignment of this MFMA is 32 js + 4 e + kb for both operands.
+// The live chunks (from the descriptor) are divided evenly among the `parts` workgroups of
+// a (kv head, pair tile); each writes one partial per pair: [M][n_heads][parts][132].
+// ---------------------------------------------------------------------------
+constexpr int kPairTile = 16;
+constexpr int kVPitch = 2 * kHd + 32;      // bytes per staged V row
+constexpr int kPPitch = 2 * kChunk + 16;   // bytes per staged P row
+constexpr int kMaxParts = 16;
+constexpr int kAttnWaves = 4;
+
+typedef __bf16 attn_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float attn_f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ attn_bf16x8_t attn_as_bf16x8(const uint4 v) {
+    attn_bf16x8_t r;
+    __builtin_memcpy(&r, &v, 16);
+    return r;
+}
+
+// live parts of a step: the live chunks split into runs of ceil(live / parts)
+__host__ __device__ inline int attn_chunks_per_part(int live_chunks, int parts) {
+    return (live_chunks + parts - 1) / parts;
+}
+
+__global__ void __launch_bounds__(kAttnWaves * 64)
+attn_mfma_kernel(const uint16_t *q, const uint16_t *k_layer, const uint16_t *v_layer,
+                 const int32_t *meta, float *part_out, float scale_log2e, int M, int n_heads,
+                 int n_kv, int G, int slots, int sigma, int parts) {
+    __shared__ __attribute__((aligned(16))) unsigned char v_lds[kChunk * kVPitch];
+    __shared__ __attribute__((aligned(16))) unsigned char p_lds[kPairTile * kPPitch];
+    __shared__ __attribute__((aligned(16))) float st_max[kAttnWaves][kPairTile];
+    __shared__ __attribute__((aligned(16))) float st_sum[kAttnWaves][kPairTile];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int col = lane & 15, kb = lane >> 4;
+    int id = blockIdx.x;
+    const int kvh = id % n_kv;
+    id /= n_kv;
+    const int part = id % parts;
+    const int pt = id / parts;
+
+    // a descriptor that does not fit the segment is clamped, never followed out of bounds
+    const int cache_len = min(max(meta[0], 0), sigma);
+    const int hide = meta[1];
+    const int total = cache_len + M;
+    const int live_chunks = (total + kChunk - 1) / kChunk;
+    const int cpw = attn_chunks_per_part(live_chunks, parts);
+    const int c_begin = part * cpw;
+    if (c_begin >= live_chunks) return;  // whole workgroup; the combine step counts the same parts
+    const int c_end = min(c_begin + cpw, live_chunks);
+    const int pairs_total = M * G;
+
+    // A operand of S: this lane's pair (tile row `col`), dims 32 j + 8 kb .. + 8
+    uint4 qreg[4];
+    {
+        const int qp = min(pt * kPairTile + col, pairs_total - 1);
+        const int qm = qp / G, qg = qp - qm * G;
+        const uint4 *qrow =
+            reinterpret_cast<const uint4 *>(q + ((size_t)qm * n_heads + kvh * G + qg) * kHd);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qreg[j] = qrow[4 * j + kb];
+    }
+    // the four pairs whose results this lane holds (D layout: tile rows 4 kb + r)
+    bool valid[4];
+    int row_of[4], head_of[4];
+    uint32_t wmask[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int pd = pt * kPairTile + 4 * kb + r;
+        valid[r] = pd < pairs_total;
+        const int pc = valid[r] ? pd : pairs_total - 1;
+        row_of[r] = pc / G;
+        head_of[r] = kvh * G + (pc - row_of[r] * G);
+        wmask[r] = (uint32_t)meta[2 + row_of[r]];
+    }
+
+    float m_run[4], l_run[4];
+    attn_f32x4_t acc_o[2];  // dims 32 w + 16 x + col
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        m_run[r] = -INFINITY;
+        l_run[r] = 0.0f;
+    }
+    acc_o[0] = acc_o[1] = attn_f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const uint16_t *kbase = k_layer + (size_t)kvh * slots * kHd;
+    const uint16_t *vbase = v_layer + (size_t)kvh * slots * kHd;
+    // One chunk's operands of this wave, as named registers (arrays of them end up in
+    // scratch memory): K of slot t0 + col, dims 32 j + 8 kb .. + 8 (the B operand of S; dead
+    // slots repeat the last live one and are masked), and the V rows of the same 16 slots,
+    // coalesced: lane = (row 4 i + kb, dims 8 col .. + 8).
+    struct ChunkRegs {
+        uint4 k0, k1, k2, k3, v0, v1, v2, v3;
+    };
+    auto load_chunk = [&](int c) {
+        const int t0 = c * kChunk + 16 * w;
+        ChunkRegs cr;
+        {
+            const int t = min(t0 + col, total - 1);
+            const int slot = t < cache_len ? t : sigma + (t - cache_len);
+            const uint4 *krow = reinterpret_cast<const uint4 *>(kbase + (size_t)slot * kHd);
+            cr.k0 = krow[kb];
+            cr.k1 = krow[4 + kb];
+            cr.k2 = krow[8 + kb];
+            cr.k3 = krow[12 + kb];
+        }
+        auto v_row = [&](int i) {
+            const int t = min(t0 + 4 * i + kb, total - 1);
+            const int slot = t < cache_len ? t : sigma + (t - cache_len);
+            return reinterpret_cast<const uint4 *>(vbase + (size_t)slot * kHd)[col];
+        };
+        cr.v0 = v_row(0);
+        cr.v1 = v_row(1);
+        cr.v2 = v_row(2);
+        cr.v3 = v_row(3);
+        return cr;
+    };
+
+    ChunkRegs cur = load_chunk(c_begin);
+    for (int c = c_begin; c < c_end; ++c) {
+        const int t0 = c * kChunk + 16 * w;  // this wave's 16 slots
+        // the next chunk's loads go out before this one is worked on (uniform branch)
+        ChunkRegs nxt = cur;
+        if (c + 1 < c_end) nxt = load_chunk(c + 1);
+        const uint4 kreg[4] = {cur.k0, cur.k1, cur.k2, cur.k3};
+        const uint4 vreg0 = cur.v0, vreg1 = cur.v1, vreg2 = cur.v2, vreg3 = cur.v3;
+
+        attn_f32x4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(attn_as_bf16x8(qreg[j]),
+                                                        attn_as_bf16x8(kreg[j]), s, 0, 0, 0);
+        // s[r]: pair 4 kb + r against slot t0 + col.  Visibility without branches: history
+        // slots but the hidden one, workspace slots by the row's bit.
+        float sc[4];
+        {
+            const int t = t0 + col;
+            const uint32_t hist_ok = (uint32_t)(t < cache_len) & (uint32_t)(t != hide);
+            const uint32_t in_ws = (uint32_t)(t >= cache_len) & (uint32_t)(t < total);
+            const int sh = (t - cache_len) & 31;
+            float mx[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t vis = (uint32_t)valid[r] & (hist_ok | (in_ws & (wmask[r] >> sh)));
+                sc[r] = (vis & 1u) ? s[r] * scale_log2e : -INFINITY;
+                mx[r] = bonsai_wave::max16(sc[r]);
+            }
+            if (col == 0)
+                *reinterpret_cast<float4 *>(&st_max[w][4 * kb]) = make_float4(mx[0], mx[1], mx[2], mx[3]);
+        }
+        __syncthreads();
+
+        float alpha[4], m_new[4];
+        {
+            const int tl = 16 * w + col;  // slot of the chunk
+            // P in A-operand order: slot 32 js + 4 e + kb' sits at index 32 js + 8 kb' + e
+            const int idx = (tl & 32) + 8 * (tl & 3) + ((tl & 31) >> 2);
+            const float4 x0 = *reinterpret_cast<const float4 *>(&st_max[0][4 * kb]);
+            const float4 x1 = *reinterpret_cast<const float4 *>(&st_max[1][4 * kb]);
+            const float4 x2 = *reinterpret_cast<const float4 *>(&st_max[2][4 * kb]);
+            const float4 x3 = *reinterpret_cast<const float4 *>(&st_max[3][4 * kb]);
+            const float mc[4] = {fmaxf(fmaxf(x0.x, x1.x), fmaxf(x2.x, x3.x)),
+                                 fmaxf(fmaxf(x0.y, x1.y), fmaxf(x2.y, x3.y)),
+                                 fmaxf(fmaxf(x0.z, x1.z), fmaxf(x2.z, x3.z)),
+                                 fmaxf(fmaxf(x0.w, x1.w), fmaxf(x2.w, x3.w))};
+            float sum[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                m_new[r] = fmaxf(m_run[r], mc[r]);
+                // nothing visible so far: the differences below are NaN and are replaced
+                const bool none = m_new[r] == -INFINITY;
+                const float a_raw = __builtin_amdgcn_exp2f(m_run[r] - m_new[r]);  // 0 at the first live chunk
+                const float p_raw = __builtin_amdgcn_exp2f(sc[r] - m_new[r]);
+                alpha[r] = none ? 1.0f : a_raw;
+                // p in [0, 1]: round to nearest even on the bits, no NaN case
+                uint32_t pu = __float_as_uint(none ? 0.0f : p_raw);
+                pu = (pu + 0x7fffu + ((pu >> 16) & 1u)) & 0xffff0000u;
+                *reinterpret_cast<uint16_t *>(p_lds + (4 * kb + r) * kPPitch + 2 * idx) =
+                    (uint16_t)(pu >> 16);
+                sum[r] = bonsai_wave::sum16(__uint_as_float(pu));
+            }
+            if (col == 0)
+                *reinterpret_cast<float4 *>(&st_sum[w][4 * kb]) =
+                    make_float4(sum[0], sum[1], sum[2], sum[3]);
+        }
+        {
+            unsigned char *vdst = v_lds + (16 * w + kb) * kVPitch + 16 * col;
+            *reinterpret_cast<uint4 *>(vdst) = vreg0;
+            *reinterpret_cast<uint4 *>(vdst + 4 * kVPitch) = vreg1;
+            *reinterpret_cast<uint4 *>(vdst + 8 * kVPitch) = vreg2;
+            *reinterpret_cast<uint4 *>(vdst + 12 * kVPitch) = vreg3;
+        }
+        __syncthreads();
+
+        {
+            const float4 y0 = *reinterpret_cast<const float4 *>(&st_sum[0][4 * kb]);
+            const float4 y1 = *reinterpret_cast<const float4 *>(&st_sum[1][4 * kb]);
+            const float4 y2 = *reinterpret_cast<const float4 *>(&st_sum[2][4 * kb]);
+            const float4 y3 = *reinterpret_cast<const float4 *>(&st_sum[3][4 * kb]);
+            const float tot[4] = {((y0.x + y1.x) + y2.x) + y3.x, ((y0.y + y1.y) + y2.y) + y3.y,
+                                  ((y0.z + y1.z) + y2.z) + y3.z, ((y0.w + y1.w) + y2.w) + y3.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                l_run[r] = l_run[r] * alpha[r] + tot[r];
+                m_run[r] = m_new[r];
+                acc_o[0][r] *= alpha[r];
+                acc_o[1][r] *= alpha[r];
+            }
+        }
+        uint4 pop[2];
+#pragma unroll
+        for (int js = 0; js < 2; ++js)
+            pop[js] = *reinterpret_cast<const uint4 *>(p_lds + col * kPPitch + 2 * (32 * js + 8 * kb));
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            const int d = 32 * w + 16 * x + col;
+#pragma unroll
+            for (int js = 0; js < 2; ++js) {
+                uint32_t wd[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int sl = 32 * js + 4 * e + kb;
+                    const uint32_t val =
+                        *reinterpret_cast<const uint16_t *>(v_lds + sl * kVPitch + 2 * d);
+                    wd[e >> 1] |= val << (16 * (e & 1));
+                }
+                const uint4 vop = make_uint4(wd[0], wd[1], wd[2], wd[3]);
+                acc_o[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    attn_as_bf16x8(pop[js]), attn_as_bf16x8(vop), acc_o[x], 0, 0, 0);
+            }
+        }
+        __syncthreads();  // the next chunk overwrites the staging areas
+        cur = nxt;
+    }
+
+    // acc_o[x][r]: pair 4 kb + r, dim 32 w + 16 x + col, unnormalised against m_run
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (valid[r]) {
+            float *dst = part_out +
+                         (((size_t)row_of[r] * n_heads + head_of[r]) * parts + part) * kPartStride;
+            dst[32 * w + col] = acc_o[0][r];
+            dst[32 * w + 16 + col] = acc_o[1][r];
+            if (w == 0 && col == 0) {
+                dst[kHd] = m_run[r];
+                dst[kHd + 1] = l_run[r];
+            }
+        }
+    }
+}
+
 // One workgroup per token: merge the chunk partials of every head, round to bf16,
 // then quantise the whole row (all heads) per token like `quant_input`.
 struct CombineArgs {
@@ -263,6 +532,7 @@ struct CombineArgs {
     int8_t *out_q;
     float *out_s;
     int M, n_heads, n_chunks, sigma;
+    int parts;  // 0: one partial per 64-slot chunk; > 0: the live chunks in that many even runs
 };
 
 constexpr int kCombineThreads = 256;
@@ -272,15 +542,19 @@ constexpr int kCombineMaxChunks = 136;  // sigma + M up to 8704 slots
 
 __global__ void __launch_bounds__(kCombineThreads)
 attn_combine_kernel(const float *ppart, const int32_t *pmeta, uint16_t *pout, int8_t *pq, float *ps,
-                    int pM, int pheads, int pchunks, int psigma) {
-    const CombineArgs a{ppart, pmeta, pout, pq, ps, pM, pheads, pchunks, psigma};
+                    int pM, int pheads, int pchunks, int psigma, int pparts) {
+    const CombineArgs a{ppart, pmeta, pout, pq, ps, pM, pheads, pchunks, psigma, pparts};
     __shared__ float wgt[kCombineMaxHeads * kCombineMaxChunks];  // becomes the chunk weights
     __shared__ float lsum[kCombineMaxHeads * kCombineMaxChunks];
     __shared__ float max_scratch[kCombineThreads / 64];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
     const int total = min(max(a.meta[0], 0), a.sigma) + a.M;
-    const int live_chunks = (total + kChunk - 1) / kChunk;
+    int live_chunks = (total + kChunk - 1) / kChunk;
+    if (a.parts > 0) {  // partials are runs of chunks: count the runs that hold live chunks
+        const int cpw = attn_chunks_per_part(live_chunks, a.parts);
+        live_chunks = (live_chunks + cpw - 1) / cpw;
+    }
     const int nvec = a.n_heads * (kHd / 8);
     const float *row = a.part + (size_t)m * a.n_heads * a.n_chunks * kPartStride;
 
@@ -749,6 +1023,7 @@ fp8_linear_kernel(const uint8_t *x, const float *x_scale, const uint8_t *w, floa
 bool g_fp8_ready[kMaxDevices];
 
 int g_rows_per_wave = 0;  // 0 = heuristic; set through bonsai_decode_set_tuning
+int g_attn_engine = 0;    // 0 = matrix-core chunk pass, 1 = VALU chunk pass
 
 int rows_per_wave(int M) {
     if (g_rows_per_wave >= 1 && g_rows_per_wave <= 4) return g_rows_per_wave < M ? g_rows_per_wave : (M < 4 ? M : 4);
@@ -798,6 +1073,10 @@ extern "C" int bonsai_qk_norm_rope_kv_write(const void *xqkv, const void *q_norm
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 
+extern "C" void bonsai_decode_set_attention_engine(int engine) {
+    g_attn_engine = engine == 1 ? 1 : 0;
+}
+
 extern "C" void bonsai_decode_set_tuning(int rows_per_wave_override) {
     g_rows_per_wave = rows_per_wave_override;
 }
@@ -835,6 +1114,15 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
     a.sigma = sigma;
     // the live length is cache_len + M <= sigma + M: chunks beyond it are never launched
     a.n_chunks = (sigma + M + kChunk - 1) / kChunk;
+    int parts = 0;  // partials per (row, head): chunks for the VALU pass, runs of chunks otherwise
+    if (g_attn_engine == 0) {
+        parts = a.n_chunks < kMaxParts ? a.n_chunks : kMaxParts;
+        const int tiles = (M * a.hpg + kPairTile - 1) / kPairTile;
+        hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_kv * parts * tiles), dim3(kAttnWaves * 64), 0, st,
+                           static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k_layer),
+                           static_cast<const uint16_t *>(v_layer), meta, a.part, a.scale_log2e, M,
+                           n_heads, n_kv, a.hpg, slots, sigma, parts);
+    } else {
     const int rw = rows_per_wave(M);
     a.row_groups = (M + rw - 1) / rw;
     const AttnArgs &launch = a;
@@ -850,19 +1138,21 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
         default: hipLaunchKernelGGL(attn_partial_kernel<4>, dim3(blocks), dim3(64), 0, st, ATTN_ARGS); break;
     }
 #undef ATTN_ARGS
+    }
     if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
     CombineArgs c;
-    c.part = launch.part;
+    c.part = a.part;
     c.meta = meta;
     c.out_bf16 = static_cast<uint16_t *>(out_bf16);
     c.out_q = out_q;
     c.out_s = out_s;
     c.M = M;
     c.n_heads = n_heads;
-    c.n_chunks = a.n_chunks;
+    c.n_chunks = parts > 0 ? parts : a.n_chunks;  // partial slots per (row, head)
     c.sigma = sigma;
+    c.parts = parts;
     hipLaunchKernelGGL(attn_combine_kernel, dim3(M), dim3(kCombineThreads), 0, st, c.part, c.meta,
-                       c.out_bf16, c.out_q, c.out_s, c.M, c.n_heads, c.n_chunks, c.sigma);
+                       c.out_bf16, c.out_q, c.out_s, c.M, c.n_heads, c.n_chunks, c.sigma, c.parts);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 

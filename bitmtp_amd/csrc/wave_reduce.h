@@ -59,6 +59,20 @@ __device__ __forceinline__ float max64(float v) {
     return lane63(v);
 }
 
+// The same first four steps alone: every lane of a 16-lane row ends with its row's result.
+__device__ __forceinline__ float max16(float v) {
+    v = fmaxf(v, partner<kXor1>(v));
+    v = fmaxf(v, partner<kXor2>(v));
+    v = fmaxf(v, partner<kHalfMirror>(v));
+    return fmaxf(v, partner<kMirror>(v));
+}
+__device__ __forceinline__ float sum16(float v) {
+    v += partner<kXor1>(v);
+    v += partner<kXor2>(v);
+    v += partner<kHalfMirror>(v);
+    return v + partner<kMirror>(v);
+}
+
 template <typename T>
 __device__ __forceinline__ T sum64(T v) {
     const int lane = (int)(threadIdx.x & 63);

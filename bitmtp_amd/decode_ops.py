@@ -44,6 +44,8 @@ def load_decode_kernel() -> None:
     lib.bonsai_decode_attention.restype = ci
     lib.bonsai_decode_set_tuning.argtypes = [ci]
     lib.bonsai_decode_set_tuning.restype = None
+    lib.bonsai_decode_set_attention_engine.argtypes = [ci]
+    lib.bonsai_decode_set_attention_engine.restype = None
     lib.bonsai_kv_commit.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
     lib.bonsai_kv_commit.restype = ci
     lib.bonsai_draft_chain.argtypes = [vp, ci, ci, ci, cf, vp, vp, vp, vp]

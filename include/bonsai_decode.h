@@ -66,6 +66,11 @@ int bonsai_qk_norm_rope_kv_write(const void *xqkv, const void *q_norm_w, const v
  * built-in heuristic.  No counterpart in the reference; results do not depend on it. */
 void bonsai_decode_set_tuning(int rows_per_wave);
 
+/* Chunk pass of the attention: 0 = matrix cores (default), 1 = the VALU form (one wave per
+ * query head and row group).  Process-wide; no counterpart in the reference; results agree
+ * to the tolerance stated below. */
+void bonsai_decode_set_attention_engine(int engine);
+
 /* Bytes of scratch `bonsai_decode_attention` needs for the given shape. */
 int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int slots);
 

@@ -3,8 +3,10 @@ one whole captured step against the CPU composition of the oracles, and the syst
 invariants of the generation loops (fast_generate.py:611-657,1151-1162).
 
 Tolerances: q/k-norm + RoPE, KV commit and the quantisation after attention are bit-exact;
-attention (bf16 inputs, fp32 online softmax on the GPU, float64 in the oracle) is compared
+attention (bf16 inputs, fp32 online softmax with the probabilities rounded to bf16 for the
+P V product as in the reference, model.py:1001; float64 throughout in the oracle) is compared
 on its bf16 output with rtol 2e-2 / atol 2e-3; whole-step logits with atol 6e-2 * max|logit|.
+Both chunk passes of the attention (matrix cores, the default, and the VALU form) are run.
 """
 import numpy as np
 import pytest
@@ -82,11 +84,18 @@ ATTN_CASES = [
     (16, 16, 8, 256, 240, "ar", 0),
     (5, 3, 1, 64, 30, "verify", 0),
     (8, 16, 8, 256, 77, "draft", 0),
+    # long segments: several chunks per workgroup of the matrix-core pass
+    (9, 16, 8, 4096, 3000, "verify", 0),
+    (1, 32, 8, 4096, 4095, "ar", 0),
+    (17, 32, 8, 4096, 1531, "draft", 9),
+    (3, 6, 2, 2048, 1100, "ar", 0),
 ]
 
 
+@pytest.mark.parametrize("engine", [0, 1])
 @pytest.mark.parametrize("M,n_heads,n_kv,sigma,cache_len,role,n_pend", ATTN_CASES)
-def test_attention_against_oracle(DO, oracle, M, n_heads, n_kv, sigma, cache_len, role, n_pend):
+def test_attention_against_oracle(DO, oracle, M, n_heads, n_kv, sigma, cache_len, role, n_pend,
+                                  engine):
     from bitmtp_amd import decode_ops, runtime
     rng = np.random.default_rng(hash((M, n_heads, sigma, cache_len)) % (2 ** 31))
     slots = sigma + 17
@@ -100,11 +109,15 @@ def test_attention_against_oracle(DO, oracle, M, n_heads, n_kv, sigma, cache_len
     out = torch.zeros(M, n_heads * 128, dtype=torch.bfloat16, device=DEV)
     out_q = torch.zeros(M, n_heads * 128, dtype=torch.int8, device=DEV)
     out_s = torch.zeros(M, dtype=torch.float32, device=DEV)
-    print(f"attention case M={M} heads={n_heads}/{n_kv} sigma={sigma} cache_len={cache_len} {role}",
-          flush=True)
-    decode_ops.decode_attention(q.to(DEV), k.to(DEV), v.to(DEV), meta, scratch, sigma,
-                                out_bf16=out, out_q=out_q, out_s=out_s)
-    torch.cuda.synchronize()
+    print(f"attention case M={M} heads={n_heads}/{n_kv} sigma={sigma} cache_len={cache_len} {role} "
+          f"engine={engine}", flush=True)
+    decode_ops.decode_lib().bonsai_decode_set_attention_engine(engine)
+    try:
+        decode_ops.decode_attention(q.to(DEV), k.to(DEV), v.to(DEV), meta, scratch, sigma,
+                                    out_bf16=out, out_q=out_q, out_s=out_s)
+        torch.cuda.synchronize()
+    finally:
+        decode_ops.decode_lib().bonsai_decode_set_attention_engine(0)
     vis = runtime.dense_visibility(desc, M, sigma)
     # the oracle reads workspace rows where the kernel does: slots sigma..sigma+M-1
     want = DO.attention(bf16_bits(q), bf16_bits(k), bf16_bits(v), vis, 1 / np.sqrt(128))
@@ -318,10 +331,16 @@ def test_captured_step_against_cpu_composition(DO, tiny, role, M, n_pend):
     want = O.bf16_bits_to_f32(want_bits)[:, : model.args.vocab_size]
     tol = 6e-2 * np.abs(want).max()
     assert np.abs(got - want).max() <= tol
-    # the KV rows the step wrote agree with the oracle's to the last place or two
+    # the K rows the step wrote: those of layer 0 do not pass through attention and agree with
+    # the oracle's to the last place or two; deeper layers carry the bf16 rounding of the
+    # attention probabilities (the reference rounds them too, the float64 oracle does not)
     new_k = bf16_bits(atlas.kv(sigma))[0][:, :, sigma:sigma + M]
-    d = np.abs(bf16_ordinal(new_k) - bf16_ordinal(kk[:, :, sigma:sigma + M]))
+    ref_k = kk[:, :, sigma:sigma + M]
+    d = np.abs(bf16_ordinal(new_k[0]) - bf16_ordinal(ref_k[0]))
     assert np.quantile(d, 0.99) <= 2
+    from oracle import oracle as O2
+    dk = np.abs(O2.bf16_bits_to_f32(new_k) - O2.bf16_bits_to_f32(ref_k))
+    assert dk.max() <= 6e-2 * np.abs(O2.bf16_bits_to_f32(ref_k)).max()
     # argmax / confidence outputs describe the logits the step produced
     wt, wc, wn = DO.draft_chain(got, atlas.threshold)
     assert toks.tolist() == wt.tolist()
