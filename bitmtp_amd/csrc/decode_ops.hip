@@ -648,6 +648,112 @@ attn_combine_kernel(const float *ppart, const int32_t *pmeta, uint16_t *pout, in
     }
 }
 
+// The same merge for the matrix-core chunk pass, whose partial count per (row, head) is at
+// most kMaxParts = 16: one workgroup of 512 threads per token, thread = (head, 8 dims).  The
+// 16 lanes of a head are one DPP row: lane j turns part j's (max, sum) into its normalised
+// weight with two row reductions, the weights travel by row_share, and every thread has
+// already requested its slice of all live partials, so the kernel is one memory round trip
+// long.  Accumulation runs over the parts in ascending order.
+constexpr int kCombinePartsThreads = 512;
+
+template <int CTRL>
+__device__ __forceinline__ float row_share(float v) {
+    const int x = __float_as_int(v);
+    return __int_as_float(__builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false));
+}
+
+__global__ void __launch_bounds__(kCombinePartsThreads)
+attn_combine_parts_kernel(const float *part, const int32_t *meta, uint16_t *out_bf16, int8_t *out_q,
+                          float *out_s, int M, int n_heads, int parts, int sigma) {
+    __shared__ float max_scratch[kCombinePartsThreads / 64];
+    const int m = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int total = min(max(meta[0], 0), sigma) + M;
+    const int live_chunks = (total + kChunk - 1) / kChunk;
+    const int cpw = attn_chunks_per_part(live_chunks, parts);
+    const int live = (live_chunks + cpw - 1) / cpw;  // <= parts <= kMaxParts
+    const int nvec = n_heads * (kHd / 8);
+    const bool mine = tid < nvec;
+    const int v = mine ? tid : nvec - 1;
+    const int head = v >> 4, j = v & 15;
+    const float *hbase = part + ((size_t)m * n_heads + head) * parts * kPartStride;
+
+    // this thread's 8 dims of every live partial, and part j's statistics
+    float4 x0[kMaxParts], x1[kMaxParts];
+#pragma unroll
+    for (int c = 0; c < kMaxParts; ++c) {
+        if (c < live) {  // uniform
+            const float4 *src = reinterpret_cast<const float4 *>(hbase + (size_t)c * kPartStride + 8 * j);
+            x0[c] = src[0];
+            x1[c] = src[1];
+        }
+    }
+    float2 ml = make_float2(-INFINITY, 0.0f);
+    if (j < live) ml = *reinterpret_cast<const float2 *>(hbase + (size_t)j * kPartStride + kHd);
+
+    const float mx = bonsai_wave::max16(ml.x);
+    const float e = (ml.x == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ml.x - mx);
+    const float den = bonsai_wave::sum16(e * ml.y);
+    const float wj = e * (den > 0.0f ? 1.0f / den : 0.0f);  // weight of part j
+
+    float num[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) num[i] = 0.0f;
+#define BONSAI_COMBINE_PART(C)                                                      \
+    {                                                                               \
+        const float wc = row_share<0x150 + (C)>(wj);                                \
+        if ((C) < live) {                                                           \
+            num[0] = fmaf(wc, x0[C].x, num[0]); num[1] = fmaf(wc, x0[C].y, num[1]); \
+            num[2] = fmaf(wc, x0[C].z, num[2]); num[3] = fmaf(wc, x0[C].w, num[3]); \
+            num[4] = fmaf(wc, x1[C].x, num[4]); num[5] = fmaf(wc, x1[C].y, num[5]); \
+            num[6] = fmaf(wc, x1[C].z, num[6]); num[7] = fmaf(wc, x1[C].w, num[7]); \
+        }                                                                           \
+    }
+    BONSAI_COMBINE_PART(0) BONSAI_COMBINE_PART(1) BONSAI_COMBINE_PART(2) BONSAI_COMBINE_PART(3)
+    BONSAI_COMBINE_PART(4) BONSAI_COMBINE_PART(5) BONSAI_COMBINE_PART(6) BONSAI_COMBINE_PART(7)
+    BONSAI_COMBINE_PART(8) BONSAI_COMBINE_PART(9) BONSAI_COMBINE_PART(10) BONSAI_COMBINE_PART(11)
+    BONSAI_COMBINE_PART(12) BONSAI_COMBINE_PART(13) BONSAI_COMBINE_PART(14) BONSAI_COMBINE_PART(15)
+#undef BONSAI_COMBINE_PART
+
+    float o[8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        o[i] = bf16_round(num[i]);
+        if (mine) amax = fmaxf(amax, fabsf(o[i]));
+    }
+    if (mine && out_bf16 != nullptr) {
+        uint4 wv;
+        wv.x = f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[1]) << 16);
+        wv.y = f32_to_bf16_bits(o[2]) | (f32_to_bf16_bits(o[3]) << 16);
+        wv.z = f32_to_bf16_bits(o[4]) | (f32_to_bf16_bits(o[5]) << 16);
+        wv.w = f32_to_bf16_bits(o[6]) | (f32_to_bf16_bits(o[7]) << 16);
+        reinterpret_cast<uint4 *>(out_bf16 + (size_t)m * nvec * 8)[v] = wv;
+    }
+    if (out_q == nullptr) return;  // uniform over the grid
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) max_scratch[tid >> 6] = amax;
+    __syncthreads();
+    amax = max_scratch[0];
+#pragma unroll
+    for (int wv = 1; wv < kCombinePartsThreads / 64; ++wv) amax = fmaxf(amax, max_scratch[wv]);
+    const float sval = (1.0f / fmaxf(amax, 1e-5f)) * 127.0f;
+    if (tid == 0) out_s[m] = sval;
+    if (mine) {
+        uint32_t b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float r = __builtin_rintf(o[i] * sval);
+            r = fminf(fmaxf(r, -128.0f), 127.0f);
+            b[i] = (uint32_t)((int)r) & 0xffu;
+        }
+        uint2 wq;
+        wq.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        wq.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+        reinterpret_cast<uint2 *>(out_q + (size_t)m * nvec * 8)[v] = wq;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // KV commit: rows [src, src+n) -> [dst, dst+n) for every (k|v, layer, kv head).
 // One thread per 16 bytes.
@@ -1151,8 +1257,14 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
     c.n_chunks = parts > 0 ? parts : a.n_chunks;  // partial slots per (row, head)
     c.sigma = sigma;
     c.parts = parts;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(M), dim3(kCombineThreads), 0, st, c.part, c.meta,
-                       c.out_bf16, c.out_q, c.out_s, c.M, c.n_heads, c.n_chunks, c.sigma, c.parts);
+    if (parts > 0)
+        hipLaunchKernelGGL(attn_combine_parts_kernel, dim3(M), dim3(kCombinePartsThreads), 0, st,
+                           c.part, c.meta, c.out_bf16, c.out_q, c.out_s, c.M, c.n_heads, parts,
+                           c.sigma);
+    else
+        hipLaunchKernelGGL(attn_combine_kernel, dim3(M), dim3(kCombineThreads), 0, st, c.part,
+                           c.meta, c.out_bf16, c.out_q, c.out_s, c.M, c.n_heads, c.n_chunks,
+                           c.sigma, c.parts);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 
