@@ -2,9 +2,12 @@
 //
 //   qk_norm_rope_kernel   split + per-head q/k RMSNorm + RoPE + KV write
 //                         (src/bonsai_sft/gpu/model.py:388-436)
-//   attn_partial_kernel   softmax(q k^T) v over one 64-slot chunk of the shared KV
-//   attn_combine_kernel   merges the chunks, rounds to bf16 and quantises per token
+//   attn_mfma_kernel      softmax(q k^T) v over a run of 64-slot chunks of the shared KV for a
+//                         tile of (row, query head) pairs, on the matrix cores
+//   attn_combine_parts_kernel   merges the runs, rounds to bf16 and quantises per token
 //                         (src/bonsai_sft/gpu/model.py:996-1005)
+//   attn_partial_kernel / attn_combine_kernel   the VALU form of the same two steps
+//                         (one wave per query head, row group and chunk), selectable
 //   kv_commit_kernel      workspace rows -> history rows (fast_runtime.py:467-508)
 //   draft_rows_kernel / draft_accept_kernel   argmax + confidence chain
 //                         (src/bonsai_sft/gpu/fast_generate.py:111-130)
@@ -13,7 +16,7 @@
 //                         1268-1275)
 //
 // Attention is HBM/L2-bound integer-free fp work: per layer it reads
-// 2 * n_kv * (cache_len + M) * 256 bytes of KV once per query-head group.  The mask
+// 2 * n_kv * (cache_len + M) * 256 bytes of KV once per tile of 16 (row, query head) pairs.  The mask
 // is not a tensor: history visibility is `slot < cache_len && slot != hide`, workspace
 // visibility one 32-bit word per row, both read from a small device descriptor, so a
 // replayed graph only touches the live part of the buffer.

@@ -82,9 +82,10 @@ int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int slots);
  *   scratch  at least bonsai_decode_attention_scratch_bytes(M, n_heads, slots) bytes
  *   out_bf16 bf16 [M, n_heads*128] or NULL
  *   out_q    int8 [M, n_heads*128] and out_s fp32 [M] (multiplier 127/absmax), or both NULL
- * softmax(q k^T * scale + mask) v per head with fp32 accumulation; the KV read is
- * bounded by cache_len + M, not by the buffer size.  Compared with a fp32 reference
- * within rtol 2e-2 / atol 2e-3 on the bf16 output (bf16 inputs, fp32 softmax). */
+ * softmax(q k^T * scale + mask) v per head with fp32 accumulation (the probabilities enter
+ * the P V product rounded to bf16, as in the reference, model.py:1001); the KV read is
+ * bounded by cache_len + M, not by the buffer size.  Compared with a float64 reference
+ * within rtol 2e-2 / atol 2e-3 on the bf16 output. */
 int bonsai_decode_attention(const void *q, const void *k_layer, const void *v_layer,
                             const int32_t *meta, void *scratch, void *out_bf16, int8_t *out_q,
                             float *out_s, float scale, int M, int n_heads, int n_kv, int slots,
