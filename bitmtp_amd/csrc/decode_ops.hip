@@ -871,6 +871,122 @@ __global__ void draft_accept_kernel(const float *conf, int rows, float threshold
     accept[1] = rows;
 }
 
+// The same statistics with a row split over `splits` workgroups (one workgroup per row is a
+// single CU evaluating 150k exponentials): partial (max, index, sum) per split into a
+// scratch buffer, then one small workgroup merges them per row and walks the chain.
+constexpr int kDraftSplitThreads = 256;
+constexpr int kDraftSplits = 32;
+
+__device__ __forceinline__ RowStat wave_merge(RowStat st) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        RowStat o;
+        o.mx = __shfl_xor(st.mx, off);
+        o.idx = __shfl_xor(st.idx, off);
+        o.sum = __shfl_xor(st.sum, off);
+        st = merge(st, o);
+    }
+    return st;
+}
+
+__global__ void __launch_bounds__(kDraftSplitThreads)
+draft_rows_split_kernel(const uint16_t *logits, int ld, int vocab, int splits, float *scratch) {
+    __shared__ RowStat wave_stat[kDraftSplitThreads / 64];
+    const int row = blockIdx.x / splits, sp = blockIdx.x % splits;
+    const int tid = threadIdx.x;
+    const uint16_t *x = logits + (size_t)row * ld;
+    RowStat st;
+    st.mx = -INFINITY;
+    st.idx = 0x7fffffff;
+    st.sum = 0.0f;
+    const int nvec = vocab / 8;
+    const int per = (nvec + splits - 1) / splits;
+    const int v_end = min(nvec, (sp + 1) * per);
+    for (int v = sp * per + tid; v < v_end; v += kDraftSplitThreads) {
+        const uint4 raw = reinterpret_cast<const uint4 *>(x)[v];
+        const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+        float e[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            e[2 * i] = bf16_bits_to_f32(d[i] & 0xffffu);
+            e[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+        }
+        float vm = e[0];
+        int vi = 0;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+            if (e[i] > vm) {
+                vm = e[i];
+                vi = i;
+            }
+        }
+        if (!(vm == vm)) continue;  // a NaN vector contributes nothing
+        const float nm = fmaxf(st.mx, vm);
+        float s = (st.mx == -INFINITY) ? 0.0f : st.sum * __builtin_amdgcn_exp2f((st.mx - nm) * 1.44269504f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += __builtin_amdgcn_exp2f((e[i] - nm) * 1.44269504f);
+        if (vm > st.mx) st.idx = v * 8 + vi;
+        st.mx = nm;
+        st.sum = s;
+    }
+    if (sp == splits - 1) {
+        for (int c = nvec * 8 + tid; c < vocab; c += kDraftSplitThreads) {  // ragged tail
+            RowStat one;
+            one.mx = bf16_bits_to_f32(x[c]);
+            one.idx = c;
+            one.sum = 1.0f;
+            if (one.mx == one.mx) st = merge(st, one);
+        }
+    }
+    st = wave_merge(st);
+    if ((tid & 63) == 0) wave_stat[tid >> 6] = st;
+    __syncthreads();
+    if (tid == 0) {
+        RowStat t = wave_stat[0];
+        for (int w = 1; w < kDraftSplitThreads / 64; ++w) t = merge(t, wave_stat[w]);
+        float *dst = scratch + (size_t)blockIdx.x * 4;
+        dst[0] = t.mx;
+        dst[1] = __int_as_float(t.idx);
+        dst[2] = t.sum;
+    }
+}
+
+__global__ void __launch_bounds__(1024)
+draft_merge_accept_kernel(const float *scratch, int rows, int splits, float threshold,
+                          int32_t *tokens, float *conf, int32_t *accept) {
+    __shared__ float conf_lds[BONSAI_MAX_WIDTH];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (int row = w; row < rows; row += 16) {  // rows <= 32: every wave runs the same two rounds at most
+        RowStat st;
+        st.mx = -INFINITY;
+        st.idx = 0x7fffffff;
+        st.sum = 0.0f;
+        if (lane < splits) {
+            const float *src = scratch + ((size_t)row * splits + lane) * 4;
+            st.mx = src[0];
+            st.idx = __float_as_int(src[1]);
+            st.sum = src[2];
+        }
+        st = wave_merge(st);
+        if (lane == 0) {
+            const float c = st.sum > 0.0f ? 1.0f / st.sum : 0.0f;
+            tokens[row] = st.idx == 0x7fffffff ? 0 : st.idx;
+            conf[row] = c;
+            conf_lds[row] = c;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int n = 1;
+        for (int r = 1; r < rows; ++r) {
+            if (!(conf_lds[r] > threshold)) break;
+            ++n;
+        }
+        accept[0] = n;
+        accept[1] = rows;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // bf16 output projection: out[m][n] = sum_k x[m][k] * w[n][k], the lm_head of a sign-weight
 // backbone (`_lm_head`, precision "bf16": F.linear(h, W), src/bonsai_sft/gpu/model.py:1296).
@@ -1296,6 +1412,27 @@ extern "C" int bonsai_draft_chain(const void *logits, int rows, int ld, int voca
                        static_cast<const uint16_t *>(logits), ld, vocab, tokens, conf);
     if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
     hipLaunchKernelGGL(draft_accept_kernel, dim3(1), dim3(64), 0, st, conf, rows, threshold, accept);
+    return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" int64_t bonsai_draft_chain_scratch_bytes(int rows) {
+    return rows < 1 ? 0 : (int64_t)rows * kDraftSplits * 4 * (int64_t)sizeof(float);
+}
+
+extern "C" int bonsai_draft_chain_ws(const void *logits, int rows, int ld, int vocab, float threshold,
+                                     int32_t *tokens, float *conf, int32_t *accept, void *scratch,
+                                     void *stream) {
+    if (!logits || !tokens || !conf || !accept || !scratch) return BONSAI_DECODE_ERR_ARG;
+    if (rows < 1 || rows > BONSAI_MAX_WIDTH || vocab < 1 || ld < vocab || ld % 8 != 0)
+        return BONSAI_DECODE_ERR_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(draft_rows_split_kernel, dim3(rows * kDraftSplits), dim3(kDraftSplitThreads), 0,
+                       st, static_cast<const uint16_t *>(logits), ld, vocab, kDraftSplits,
+                       static_cast<float *>(scratch));
+    if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
+    hipLaunchKernelGGL(draft_merge_accept_kernel, dim3(1), dim3(1024), 0, st,
+                       static_cast<const float *>(scratch), rows, kDraftSplits, threshold, tokens,
+                       conf, accept);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 

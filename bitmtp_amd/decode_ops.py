@@ -50,6 +50,10 @@ def load_decode_kernel() -> None:
     lib.bonsai_kv_commit.restype = ci
     lib.bonsai_draft_chain.argtypes = [vp, ci, ci, ci, cf, vp, vp, vp, vp]
     lib.bonsai_draft_chain.restype = ci
+    lib.bonsai_draft_chain_ws.argtypes = [vp, ci, ci, ci, cf, vp, vp, vp, vp, vp]
+    lib.bonsai_draft_chain_ws.restype = ci
+    lib.bonsai_draft_chain_scratch_bytes.argtypes = [ci]
+    lib.bonsai_draft_chain_scratch_bytes.restype = ctypes.c_int64
     lib.bonsai_bf16_linear.argtypes = [vp, vp, vp, ci, ci, ci, vp]
     lib.bonsai_bf16_linear.restype = ci
     lib.bonsai_fp8_quant_rows.argtypes = [vp, vp, vp, ci, ci, vp]
@@ -172,7 +176,8 @@ def kv_commit(kv: torch.Tensor, src_slot: int, dst_slot: int, n: int) -> None:
 
 
 def draft_chain(logits: torch.Tensor, vocab: int, threshold: float, tokens: torch.Tensor,
-                conf: torch.Tensor, accept: torch.Tensor) -> None:
+                conf: torch.Tensor, accept: torch.Tensor,
+                scratch: Optional[torch.Tensor] = None) -> None:
     """Row argmax, confidence ``exp(max - logsumexp)`` and the accepted-prefix length
     ``1 + longest prefix of rows 1.. with conf > threshold`` (reference:
     fast_generate.py:111-130).  ``logits`` bf16 ``[rows, ld]``; outputs are pre-allocated
@@ -185,9 +190,18 @@ def draft_chain(logits: torch.Tensor, vocab: int, threshold: float, tokens: torc
     _need(tokens.numel() >= rows and conf.numel() >= rows and accept.numel() >= 2,
           "draft_chain output buffers too small")
     with torch.cuda.device(logits.device):
-        rc = decode_lib().bonsai_draft_chain(_ptr(logits), rows, ld, int(vocab), float(threshold),
-                                             _ptr(tokens), _ptr(conf), _ptr(accept),
-                                             _stream(logits.device))
+        if scratch is not None:
+            # rows split over several workgroups, partial statistics through `scratch`
+            need = int(decode_lib().bonsai_draft_chain_scratch_bytes(rows))
+            _need(scratch.is_cuda and scratch.is_contiguous()
+                  and scratch.numel() * scratch.element_size() >= need, "draft_chain scratch too small")
+            rc = decode_lib().bonsai_draft_chain_ws(_ptr(logits), rows, ld, int(vocab),
+                                                    float(threshold), _ptr(tokens), _ptr(conf),
+                                                    _ptr(accept), _ptr(scratch), _stream(logits.device))
+        else:
+            rc = decode_lib().bonsai_draft_chain(_ptr(logits), rows, ld, int(vocab), float(threshold),
+                                                 _ptr(tokens), _ptr(conf), _ptr(accept),
+                                                 _stream(logits.device))
     _need(rc == 0, f"bonsai_draft_chain failed with status {rc}")
 
 

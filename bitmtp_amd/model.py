@@ -526,4 +526,6 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
               "bonsai_add_rmsnorm_quant_int8")
         logits = ws.logits_view(rows, model.head_rows)
         _gemv(ws.l_q, ws.l_s, model.head, logits, rows, stream)
-    decode_ops.draft_chain(logits, args.vocab_size, threshold, io.tokens_out, io.conf, io.accept)
+    # (the attention scratch is free again by now and far larger than the chain needs)
+    decode_ops.draft_chain(logits, args.vocab_size, threshold, io.tokens_out, io.conf, io.accept,
+                           scratch=ws.attn_scratch)

@@ -109,6 +109,16 @@ int bonsai_kv_commit(void *kv, int n_layers, int n_kv, int slots, int src_slot, 
 int bonsai_draft_chain(const void *logits, int rows, int ld, int vocab, float threshold,
                        int32_t *tokens, float *conf, int32_t *accept, void *stream);
 
+/* The same chain with every row split over several workgroups (one workgroup per row is a
+ * single CU working through the whole vocabulary): partial statistics go through `scratch`
+ * (at least bonsai_draft_chain_scratch_bytes(rows) bytes of device memory, contents
+ * undefined afterwards; rows <= BONSAI_MAX_WIDTH).  Same outputs; the confidence may differ
+ * from the one-workgroup form in the last place (another summation order). */
+int64_t bonsai_draft_chain_scratch_bytes(int rows);
+int bonsai_draft_chain_ws(const void *logits, int rows, int ld, int vocab, float threshold,
+                          int32_t *tokens, float *conf, int32_t *accept, void *scratch,
+                          void *stream);
+
 /* bf16 output projection of a sign-weight (Q1) backbone, whose graphs keep the tied lm_head
  * in bf16: logits = F.linear(h, W) (`_lm_head`, precision "bf16",
  * src/bonsai_sft/gpu/model.py:1296; chosen in src/bonsai_sft/gpu/fast_runtime.py:175-178).

@@ -176,15 +176,23 @@ def test_draft_chain_kernel(DO, rows, vocab, ld):
         logits[2, 5] = 25.0
         logits[2, 17] = 25.0
     logits[:, vocab:] = 100.0
-    tokens = torch.zeros(rows, dtype=torch.int32, device=DEV)
-    conf = torch.zeros(rows, dtype=torch.float32, device=DEV)
-    accept = torch.zeros(2, dtype=torch.int32, device=DEV)
-    decode_ops.draft_chain(logits.to(DEV), vocab, 0.9, tokens, conf, accept)
-    torch.cuda.synchronize()
     wt, wc, wn = DO.draft_chain(logits[:, :vocab].float().numpy(), 0.9)
-    assert tokens.cpu().tolist() == wt.tolist()
-    np.testing.assert_allclose(conf.cpu().numpy(), wc, rtol=2e-3, atol=1e-6)
-    assert accept.cpu().tolist() == [wn, rows]
+    # one workgroup per row, and the rows split over several workgroups through a scratch buffer
+    nbytes = int(decode_ops.decode_lib().bonsai_draft_chain_scratch_bytes(rows))
+    assert nbytes == rows * 32 * 16
+    for scratch in (None, torch.full((nbytes // 4,), float("nan"), device=DEV)):
+        tokens = torch.zeros(rows, dtype=torch.int32, device=DEV)
+        conf = torch.zeros(rows, dtype=torch.float32, device=DEV)
+        accept = torch.zeros(2, dtype=torch.int32, device=DEV)
+        print(f"[case] draft_chain rows={rows} vocab={vocab} split={scratch is not None}", flush=True)
+        decode_ops.draft_chain(logits.to(DEV), vocab, 0.9, tokens, conf, accept, scratch=scratch)
+        torch.cuda.synchronize()
+        assert tokens.cpu().tolist() == wt.tolist()
+        np.testing.assert_allclose(conf.cpu().numpy(), wc, rtol=2e-3, atol=1e-6)
+        assert accept.cpu().tolist() == [wn, rows]
+    with pytest.raises(RuntimeError):
+        decode_ops.draft_chain(logits.to(DEV), vocab, 0.9, tokens, conf, accept,
+                               scratch=torch.zeros(4, device=DEV))
 
 
 # ---------------------------------------------------------------- bf16 output projection
