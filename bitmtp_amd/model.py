@@ -393,6 +393,7 @@ class StepIO:
     out: torch.Tensor            # int32 [2M+2] device
     out_host: torch.Tensor       # pinned mirror
     uploaded: "torch.cuda.Event"  # recorded after each upload of step_in_host
+    downloaded: bool = False      # the last replay already copied `out` into `out_host`
 
     @property
     def meta(self) -> torch.Tensor:

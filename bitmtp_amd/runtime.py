@@ -278,9 +278,14 @@ class GraphAtlas:
                 run()  # warm-up outside capture: lazy library set-up happens here
             torch.cuda.current_stream(self.device).wait_stream(side)
             torch.cuda.synchronize(self.device)
+            # the graph carries its own upload of the step inputs and download of the results
+            # (copy nodes between the pinned mirrors and the device vectors): a replay is one
+            # launch call on the host
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
+                io.step_in.copy_(io.step_in_host, non_blocking=True)
                 run()
+                io.out_host.copy_(io.out, non_blocking=True)
         cg = CapturedGraph(graph=graph, io=io, M=M, sigma=sigma, role=role, P=M - self.D,
                            logits_start=ls, logits_end=le)
         cg._eager = run
@@ -302,18 +307,23 @@ class GraphAtlas:
         host[: 2 + M] = desc
         host[2 + M: 2 + 2 * M] = positions
         host[2 + 2 * M:] = tokens
-        g.io.step_in.copy_(g.io.step_in_host, non_blocking=True)
-        g.io.uploaded.record(torch.cuda.current_stream(self.device))
+        stream = torch.cuda.current_stream(self.device)
         if g.graph is not None:
-            g.graph.replay()
+            g.graph.replay()          # uploads, runs the step, downloads the results
+            g.io.uploaded.record(stream)
+            g.io.downloaded = True
         else:
+            g.io.step_in.copy_(g.io.step_in_host, non_blocking=True)
+            g.io.uploaded.record(stream)
             g._eager()
+            g.io.downloaded = False
         self.replays += 1
 
     def read_outputs(self, g: CapturedGraph) -> Tuple[np.ndarray, np.ndarray, int]:
         """One device-to-host copy + synchronisation: (argmax tokens, confidences,
         device-side accepted-prefix length) of the projected rows."""
-        g.io.out_host.copy_(g.io.out, non_blocking=True)
+        if not g.io.downloaded:
+            g.io.out_host.copy_(g.io.out, non_blocking=True)
         torch.cuda.current_stream(self.device).synchronize()
         rows = g.logits_end - g.logits_start
         out = g.io.out_host.numpy()
