@@ -322,9 +322,15 @@ class GraphAtlas:
     def read_outputs(self, g: CapturedGraph) -> Tuple[np.ndarray, np.ndarray, int]:
         """One device-to-host copy + synchronisation: (argmax tokens, confidences,
         device-side accepted-prefix length) of the projected rows."""
-        if not g.io.downloaded:
+        if g.io.downloaded:
+            # the event after the replay: polling it returns sooner than a blocking
+            # synchronisation wakes the thread up
+            ev = g.io.uploaded
+            while not ev.query():
+                pass
+        else:
             g.io.out_host.copy_(g.io.out, non_blocking=True)
-        torch.cuda.current_stream(self.device).synchronize()
+            torch.cuda.current_stream(self.device).synchronize()
         rows = g.logits_end - g.logits_start
         out = g.io.out_host.numpy()
         toks = out[:rows].copy()
