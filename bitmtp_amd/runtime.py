@@ -37,6 +37,12 @@ ROLES = ("draft", "verify", "ar")
 # ---------------------------------------------------------------------------
 # Visibility descriptors (host side, pure Python: unit-tested without a GPU)
 # ---------------------------------------------------------------------------
+def _as_int32(mask: int) -> int:
+    """A 32-bit visibility word as the signed value an int32 buffer holds (bit 31 = row 31)."""
+    mask &= 0xFFFFFFFF
+    return mask - (1 << 32) if mask >= (1 << 31) else mask
+
+
 def draft_row_masks(M: int, D: int, n_pend: int) -> List[int]:
     """Workspace visibility of a draft step (reference template:
     ``_build_mask_template``, fast_runtime.py:345-372).
@@ -56,13 +62,13 @@ def draft_row_masks(M: int, D: int, n_pend: int) -> List[int]:
     for r in range(P, M):
         block = ((1 << (r - P + 1)) - 1) << P
         masks[r] = block | earlier
-    return masks
+    return [_as_int32(m) for m in masks]
 
 
 def causal_row_masks(M: int) -> List[int]:
     """AR-causal workspace visibility of verify / AR steps: row r sees rows 0..r
     (reference: ``_build_verify_templates``, fast_runtime.py:423-441)."""
-    return [(1 << (r + 1)) - 1 for r in range(M)]
+    return [_as_int32((1 << (r + 1)) - 1) for r in range(M)]
 
 
 # output projection of each role: the backbone's own ("native"), the FP8 or the raw bf16
@@ -137,7 +143,7 @@ class GraphAtlas:
                  m_set: Tuple[int, ...] = DEFAULT_M_SET,
                  roles: Tuple[str, ...] = ROLES,
                  threshold: float = 0.9,
-                 prefill_width: int = 16,
+                 prefill_width: int = 32,
                  use_graphs: bool = True):
         contracts.validate_graph_roles(roles)
         self.model = model

@@ -84,6 +84,7 @@ ATTN_CASES = [
     (16, 16, 8, 256, 240, "ar", 0),
     (5, 3, 1, 64, 30, "verify", 0),
     (8, 16, 8, 256, 77, "draft", 0),
+    (32, 16, 8, 256, 100, "ar", 0),
     # long segments: several chunks per workgroup of the matrix-core pass
     (9, 16, 8, 4096, 3000, "verify", 0),
     (1, 32, 8, 4096, 4095, "ar", 0),
@@ -98,7 +99,7 @@ def test_attention_against_oracle(DO, oracle, M, n_heads, n_kv, sigma, cache_len
                                   engine):
     from bitmtp_amd import decode_ops, runtime
     rng = np.random.default_rng(hash((M, n_heads, sigma, cache_len)) % (2 ** 31))
-    slots = sigma + 17
+    slots = sigma + max(17, M)
     q = _rand_bf16(rng, (M, n_heads, 128), 1.5)
     k = _rand_bf16(rng, (n_kv, slots, 128), 1.5)
     v = _rand_bf16(rng, (n_kv, slots, 128), 1.0)
@@ -414,6 +415,21 @@ def test_hybrid_with_exact_verification_reproduces_ar(tiny):
     assert st["decode_tokens"] == 1 + st["accepted_drafts"] + st["verifier_bonus_tokens"]
 
 
+def test_prefill_width_does_not_change_the_tokens(tiny):
+    """The prompt may be prefilled 16 or 32 rows at a time (AR-causal replays of the same
+    kernels): the greedy continuation is the same."""
+    from bitmtp_amd import generate
+    from bitmtp_amd.runtime import GraphAtlas
+    model, atlas = tiny
+    assert atlas.prefill_width == 32
+    narrow = GraphAtlas(model, segment_ladder=(64, 256), prefill_width=16)
+    rng = np.random.default_rng(53)
+    prompt = rng.integers(0, 1000, 45).tolist()
+    a, _ = generate.ar_generate(atlas, prompt, max_gen_len=12)
+    b, _ = generate.ar_generate(narrow, prompt, max_gen_len=12)
+    assert a == b
+
+
 def test_speculative_decode_always_verifies(tiny):
     """fast_generate.py:664-899: draft + verify every iteration; with the exact width-1
     verifier the tokens are the AR ones, with the width-(D+1) verifier every committed
@@ -501,7 +517,7 @@ def test_segment_migration_keeps_the_sequence(tiny):
     decoding on from there gives the same tokens as staying put."""
     from bitmtp_amd import generate
     model, atlas = tiny
-    prompt = list(range(11, 45))
+    prompt = list(range(11, 29))
     ar, _ = generate.ar_generate(atlas, prompt, max_gen_len=12)       # lives in segment 64
     assert atlas.select_segment(len(prompt) + 12 + atlas.M_max) == 64
     # replay the same decode by hand, migrating 64 -> 256 after four tokens

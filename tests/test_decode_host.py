@@ -98,6 +98,19 @@ def test_draft_template_rows_follow_the_specification():
     assert vis[:, :cache_len].all() and not vis[:, cache_len:sigma].any()
 
 
+def test_widest_step_fits_the_32_bit_row_words():
+    """32 rows use bit 31 of the visibility word: the descriptor stays an int32 vector."""
+    for role, n_pend in (("ar", 0), ("draft", 24), ("verify", 0)):
+        desc = R.step_descriptor(role, 32, 8, 40, n_pend)
+        arr = np.array(desc, dtype=np.int32)          # raises if a word does not fit
+        assert arr.shape == (34,)
+        vis = R.dense_visibility(desc, 32, 64)
+        assert vis[31, 64 + 31] and vis.shape == (32, 96)
+    causal = R.dense_visibility(R.step_descriptor("ar", 32, 8, 40), 32, 64)
+    assert np.array_equal(causal[:, 64:], np.tril(np.ones((32, 32), dtype=bool)))
+    assert np.array_equal(causal, DO.dense_mask_causal(32, 64, 40, "ar"))
+
+
 def test_unknown_role_and_bad_pending_are_rejected():
     with pytest.raises(ValueError, match="unsupported graph role"):
         R.step_descriptor("verify_q1", 9, 8, 3, 1)
