@@ -392,7 +392,8 @@ class StepIO:
     step_in_host: torch.Tensor   # pinned mirror
     out: torch.Tensor            # int32 [2M+2] device
     out_host: torch.Tensor       # pinned mirror
-    uploaded: "torch.cuda.Event"  # recorded after each upload of step_in_host
+    uploaded: "torch.cuda.Event"  # recorded once step_in_host has been consumed: after the
+                                  # eager upload, or after the replay of a graph that carries it
     downloaded: bool = False      # the last replay already copied `out` into `out_host`
 
     @property
