@@ -48,11 +48,13 @@ def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens
     prompt = rng.integers(0, args.vocab_size, prompt_len).tolist()
 
     def best(fn):
-        res = None
+        res, prefill = None, None
         for _ in range(repeats + 1):   # the first pass also captures the graphs it needs
             out, st = fn()
+            prefill = st["prefill_time"] if prefill is None else min(prefill, st["prefill_time"])
             if res is None or st["decode_time"] < res[1]["decode_time"]:
                 res = (out, st)
+        res[1]["prefill_time"] = prefill   # the fastest prefill seen (capture excluded)
         return res
 
     out_ar, st_ar = best(lambda: ar_generate(atlas, prompt, max_gen_len=new_tokens))
