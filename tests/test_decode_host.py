@@ -314,3 +314,32 @@ def test_attention_oracle_equals_torch_sdpa():
         qq, kk, vv, attn_mask=torch.from_numpy(vis)[None, None])
     want = want[0].permute(1, 0, 2).reshape(M, -1).numpy()
     np.testing.assert_allclose(got, want, rtol=1e-9, atol=1e-12)
+
+
+def test_graph_capture_runs_with_the_garbage_collector_off():
+    """A collector run inside a stream capture can destroy another atlas's graphs and abort
+    the process: `_capture_one` collects first and keeps the collector off until the capture
+    has ended, also when the capture raises."""
+    import gc
+    atlas = R.GraphAtlas.__new__(R.GraphAtlas)
+    seen = []
+
+    def fake_impl(M, sigma, role):
+        seen.append((gc.isenabled(), torch.is_inference_mode_enabled()))
+        if role == "boom":
+            raise RuntimeError("capture failed")
+        return "graph"
+    atlas._capture_one_impl = fake_impl
+    assert gc.isenabled()
+    with torch.inference_mode():
+        assert atlas._capture_one(1, 64, "ar") == "graph"
+    assert seen == [(False, False)] and gc.isenabled()
+    with pytest.raises(RuntimeError, match="capture failed"):
+        atlas._capture_one(1, 64, "boom")
+    assert gc.isenabled()
+    gc.disable()
+    try:
+        atlas._capture_one(1, 64, "ar")
+        assert not gc.isenabled()      # a caller's own setting is left alone
+    finally:
+        gc.enable()
