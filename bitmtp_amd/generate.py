@@ -138,12 +138,11 @@ def ar_generate(atlas: GraphAtlas, input_ids: Sequence[int], max_gen_len: int = 
     eos_set = set(int(e) for e in eos_ids)
     prompt = [int(t) for t in input_ids]
     seq_len = len(prompt)
-    dev = atlas.device
     t0 = time.time()
     sigma = atlas.select_segment(seq_len + max_gen_len + atlas.M_max)
     next_tok = prefill(atlas, prompt, sigma)
     cache_len = seq_len
-    torch.cuda.synchronize(dev)
+    atlas.synchronize()
     prefill_time = time.time() - t0
     if eos_set and next_tok in eos_set:
         st = _stats_common(prefill_time, 1e-9, prefill_time, seq_len, 0)
@@ -169,7 +168,7 @@ def ar_generate(atlas: GraphAtlas, input_ids: Sequence[int], max_gen_len: int = 
         gen.append(next_tok)
         if cache_len + 1 > atlas.segment_ladder[-1]:
             break
-    torch.cuda.synchronize(dev)
+    atlas.synchronize()
     decode_time = max(time.time() - t1, 1e-9)
     st = _stats_common(prefill_time, decode_time, time.time() - t0, seq_len, len(gen))
     st.update({"n_iters": len(gen), "avg_accept": 1.0})
@@ -223,7 +222,6 @@ def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: floa
     args = atlas.args
     D = args.block_size
     MASK = args.mask_token_id
-    dev = atlas.device
     if hybrid_m is None:
         hybrid_m = default_hybrid_m(D)
     eos_set = set(int(e) for e in eos_ids)
@@ -235,7 +233,7 @@ def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: floa
     sigma = atlas.select_segment(seq_len + max_gen_len + atlas.M_max)
     next_tok = prefill(atlas, prompt, sigma)
     cache_len = seq_len
-    torch.cuda.synchronize(dev)
+    atlas.synchronize()
     prefill_time = time.time() - t0
     if eos_set and next_tok in eos_set:
         st = _stats_common(prefill_time, 1e-9, prefill_time, seq_len, 0)
@@ -336,7 +334,7 @@ def hybrid_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: floa
         if cache_len + len(pending) + D > atlas.segment_ladder[-1]:
             break
 
-    torch.cuda.synchronize(dev)
+    atlas.synchronize()
     decode_time = max(time.time() - t1, 1e-9)
     n_out = len(gen)
     if drafted_total != D * draft_iters:
@@ -414,7 +412,7 @@ def confidence_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: 
     (``create_sdlm_attention_mask``, model.py:462-505)."""
     role = draft_role(atlas, use_fp8_draft, use_bf16_draft)
     args = atlas.args
-    D, MASK, dev = args.block_size, args.mask_token_id, atlas.device
+    D, MASK = args.block_size, args.mask_token_id
     eos_set = set(int(e) for e in eos_ids)
     prompt = [int(t) for t in input_ids]
     seq_len = len(prompt)
@@ -428,7 +426,7 @@ def confidence_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: 
                  [seq_len - 1 + i for i in range(D)], cache_len, n_pend=0)
     toks, conf, _ = atlas.read_outputs(g1)
     accepted, _, eos_found = confidence_accept(toks, conf, threshold, eos_set, D)
-    torch.cuda.synchronize(dev)
+    atlas.synchronize()
     prefill_time = time.time() - t0
 
     gen: List[int] = list(accepted[:max_gen_len])
@@ -470,7 +468,7 @@ def confidence_generate(atlas: GraphAtlas, input_ids: Sequence[int], threshold: 
         eos_found = eos_hit
         if cache_len + n_pend + D > atlas.segment_ladder[-1]:
             break
-    torch.cuda.synchronize(dev)
+    atlas.synchronize()
     decode_time = max(time.time() - t1, 1e-9)
     n_out = len(gen)
     st = {

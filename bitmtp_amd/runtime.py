@@ -175,6 +175,10 @@ class GraphAtlas:
         self.graphs: Dict[Tuple[int, int, str], CapturedGraph] = {}
         self.replays = 0
 
+    def synchronize(self) -> None:
+        """Wait for everything queued on the atlas's device (the loops' timing fences)."""
+        torch.cuda.synchronize(self.device)
+
     # -- KV ------------------------------------------------------------------
     def kv(self, sigma: int) -> torch.Tensor:
         """Shared buffer of segment sigma, allocated on first use
