@@ -125,11 +125,12 @@ __global__ void __launch_bounds__(kThreads) act_quant_kernel(const void *x, int8
 // is one memory round trip plus two workgroup reductions long.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+// round to nearest even through the hardware conversion (v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+    const __bf16 b = static_cast<__bf16>(f);
+    uint16_t u;
+    __builtin_memcpy(&u, &b, 2);
+    return u;
 }
 __device__ __forceinline__ float bf16_round(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
@@ -312,7 +313,11 @@ silu_mul_quant_kernel(const uint16_t *gu, int8_t *q, float *s, int F, int T) {
         unpack8_bf16(ur[i], u);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float sg = bf16_round(g[e] / (1.0f + expf(-g[e])));
+            // silu through the hardware exp2 and reciprocal (about 1e-6 relative error, far
+            // below the bf16 rounding that follows): one CU evaluates a whole token row, and
+            // libm's expf and the IEEE division made this kernel compute-bound
+            const float ex = __builtin_amdgcn_exp2f(g[e] * -1.44269504088896341f);
+            const float sg = bf16_round(g[e] * __builtin_amdgcn_rcpf(1.0f + ex));
             nf[i][e] = bf16_round(sg * u[e]);
             if (v < nvec) amax = fmaxf(amax, fabsf(nf[i][e]));
         }
