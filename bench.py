@@ -10,7 +10,9 @@ distinct random layers larger than the 256 MB Infinity Cache, so the weights com
 from HBM, and the steps are replayed from one HIP graph so that the Python launch
 cost is outside the measurement, as in the reference's graph-replayed decode.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).
+Prints ONE JSON line: the driver's fields (metric, value, unit, ...), `config` with the
+per-width, merged-shape, lm_head and end-to-end decode figures, `roofline` of the slowest
+layer kernel and `cpu_baseline`.
 """
 from __future__ import annotations
 
@@ -286,6 +288,39 @@ def main() -> int:
         }
         del g
 
+    # the same layer bytes in the four merged matrices the decode step launches
+    # (q|k|v and gate|up concatenated along N, as the reference's prepare_merged_weights,
+    # model.py:931-956,1042-1051): 4 launches per layer instead of 7
+    merged_shapes = ((4096, 2048, (0, 1, 2)), (2048, 2048, (3,)), (12288, 2048, (4, 5)),
+                     (2048, 6144, (6,)))
+    mpool = [[(torch.cat([layer[i][0] for i in idx]).contiguous(),
+               torch.cat([layer[i][1] for i in idx]).contiguous())
+              for _, _, idx in merged_shapes] for layer in pool]
+    mouts = {(m, j): torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+             for m in WIDTHS for j, (n, _, _) in enumerate(merged_shapes)}
+    merged = {}
+    for m in WIDTHS:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            spc = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for st in range(args.steps):
+                layer = mpool[st % len(mpool)]
+                for j, (n, k, _) in enumerate(merged_shapes):
+                    q, s_ = acts[(m, k)]
+                    run.fn(q.data_ptr(), layer[j][0].data_ptr(), mouts[(m, j)].data_ptr(),
+                           s_.data_ptr(), layer[j][1].data_ptr(), m, n, k, spc)
+        g.replay()
+        torch.cuda.synchronize()
+        t = min(run.time_graph(g) for _ in range(3))
+        merged[str(m)] = {
+            "gbps": round(LAYER_BYTES * args.steps / t / 1e9, 1),
+            "pct_hbm_peak": round(LAYER_BYTES * args.steps / t / 1e9 / HBM_PEAK_GBPS * 100, 2),
+            "us_per_layer": round(t / args.steps * 1e6, 3),
+            "us_per_launch": round(t / (args.steps * len(merged_shapes)) * 1e6, 3),
+        }
+        del g
+    del mpool
+
     # secondary figure: the same 21 launches per step on four forked streams of one graph
     # (two launches may write the same output buffer at once: the values are not used)
     run.cursor = 0
@@ -374,6 +409,7 @@ def main() -> int:
             "pct_hbm_peak": round(gbps / HBM_PEAK_GBPS * 100, 2),
             "per_width": {str(m): per_width[m] for m in WIDTHS},
             "timing": "one HIP graph of all steps, HIP events on the launch stream, best of 3 replays",
+            "merged_decode_shapes_4_launches_per_layer": merged,
             "concurrent_streams": concurrent,
             "lm_head_151936x2048": head,
             "decode_1p7b_d8": decode,

@@ -403,7 +403,8 @@ size_t lds_bytes(int mt, int C) {
 // Picks lanes-per-row, workgroup size and passes for a shape.  The aim is to
 // have every lane issue a few 16-byte loads at once and enough waves (a few per
 // SIMD over 256 CUs) for the launch to cover the chip, without leaving more
-// than a quarter of the lanes past the end of short rows.
+// than about a quarter of the lanes past the end of short rows.  The constants
+// come from sweeps over the decode shapes of the 1.7B- and 4B-shaped models.
 template <int BITS>
 Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
     using F = Fmt<BITS>;
@@ -426,7 +427,11 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
         int best = 0;
         for (int cand = min_lpr; cand <= 64; cand *= 2) {
             const int it = (C + cand - 1) / cand;
-            const bool low_waste = (long)it * cand * 4 <= (long)C * 5;  // <= 25 % idle lanes
+            // idle lanes: up to 27 % of a row's slots; a whole wave per row (two extra
+            // cross-lane steps in the row reduction) only where that leaves each lane
+            // exactly two loads, then up to 34 %
+            const bool low_waste = cand < 64 ? (long)it * cand * 100 <= (long)C * 127
+                                             : (it == 2 && (long)it * cand * 100 <= (long)C * 134);
             if (!low_waste && best != 0) continue;
             best = cand;
             const long waves = ((long)N * cand + 63) / 64;
@@ -437,12 +442,18 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
     g.lpr_log2 = ilog2(lpr);
     // loads per batch: the largest of 4, 2, 1 that wastes no load slot, 4 for long rows
     const int it = (C + lpr - 1) / lpr;
-    g.batch_index = (it % 4 == 0 || it >= 8) ? 2 : (it % 2 == 0 ? 1 : 0);
+    // (one token of 2-bit weights: two at a time also for odd counts, the spare slot re-reads
+    // the last chunk)
+    const bool pair_odd = BITS == 2 && g.mt == 1 && it >= 3;
+    g.batch_index = (it % 4 == 0 || it >= 8) ? 2 : ((it % 2 == 0 || pair_odd) ? 1 : 0);
     if (g.batch_index > max_batch_index(g.mt)) g.batch_index = max_batch_index(g.mt);
     const int rpw = 64 >> g.lpr_log2;
     const long wave_passes = ((long)N + rpw - 1) / rpw;
 
-    g.waves = tu.waves_per_wg ? tu.waves_per_wg : 4;
+    // eight waves share one staging of the token tile where the rows are few, as long as
+    // that leaves at least 128 workgroups
+    g.waves = tu.waves_per_wg ? tu.waves_per_wg
+                              : ((N <= 6144 && wave_passes >= 8 * 128) ? 8 : 4);
     if (g.waves * 64 > kMaxThreads) g.waves = kMaxThreads / 64;
     g.passes = tu.passes;
     if (g.passes == 0) {
