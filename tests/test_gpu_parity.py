@@ -57,6 +57,19 @@ def test_small_shapes(oracle, bits, M, N, K):
 
 
 @pytest.mark.parametrize("bits", [2, 1])
+def test_random_shapes(oracle, bits):
+    """Forty seeded random (M, N, K): every width 1..17, ragged N, every K that is a multiple
+    of 128 up to 9728 -- whatever kernel and geometry the dispatcher picks for them."""
+    rng = np.random.default_rng(2024 + bits)
+    for i in range(40):
+        M = int(rng.integers(1, 18))
+        N = int(rng.integers(1, 600))
+        K = 128 * int(rng.integers(1, 77))
+        p = oracle.synth_problem(5000 + i, M, N, K, bits)
+        check_problem(oracle, p, bits, f"random {i}")
+
+
+@pytest.mark.parametrize("bits", [2, 1])
 def test_arbitrary_bytes_and_extreme_activations(oracle, bits):
     """Every byte value (T2 code 0 -> -2 included) and activations over all of int8."""
     rng = np.random.default_rng(7)
