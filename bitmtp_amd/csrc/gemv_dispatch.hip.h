@@ -76,11 +76,33 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
         else
             ks = (N <= 4096 && ntiles >= 4) ? 4 : ((N <= 16384 && ntiles >= 2) ? 2 : 1);
     }
-    if (ks != 1 && ks != 2 && ks != 4 && !(ks == 8 && direct)) ks = 1;
+    // Tile counts that are no power of two (K = 2560, 6144, 9728 ...) on matrices of at most
+    // 4096 rows (about one workgroup per CU: with more workgroups this form measured slower
+    // than a split of four): the direct kernel in its one-slice-per-wave form, one tile per
+    // wave up to twelve waves.  A tuning override of the split in 3..12 other than 4 and 8
+    // selects this form as well.
+    bool flex = false;
+    if (direct && (tu.row_tiles == 0 || tu.row_tiles == 1)) {
+        if (tu.k_split == 0 && (ntiles & (ntiles - 1)) != 0 && ntiles >= 3) {
+            if (N <= 4096) {
+                flex = true;
+                ks = ntiles < kMfmaFlexMaxWaves ? ntiles : kMfmaFlexMaxWaves;
+            }
+        } else if (tu.k_split >= 3 && tu.k_split <= kMfmaFlexMaxWaves && tu.k_split != 4 &&
+                   tu.k_split != 8 && tu.k_split <= ntiles) {
+            flex = true;
+            ks = tu.k_split;
+        }
+    }
+    if (!flex && ks != 1 && ks != 2 && ks != 4 && !(ks == 8 && direct)) ks = 1;
     // slices may be uneven (tile t goes to slice floor-partition): every wave still reaches the
     // single barrier after its K loop; an empty slice is never scheduled
     if (ks > ntiles) ks = 1;
     if (ks == 8) nw = 8;
+    if (flex) {
+        nw = ks;
+        R = 1;
+    }
     if (R == 0) {
         const long wgs1 = ((long)N + 16 * (nw / ks) - 1) / (16 * (nw / ks));  // workgroups at R = 1
         R = wgs1 >= 8192 ? 4 : (wgs1 >= 2048 ? 2 : 1);
@@ -111,7 +133,7 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
     args.N = N;
     args.K = K;
     args.mt = mt;
-    args.ks_log2 = ks == 8 ? 3 : (ks == 4 ? 2 : (ks == 2 ? 1 : 0));
+    args.ks_log2 = flex ? ks : (ks == 8 ? 3 : (ks == 4 ? 2 : (ks == 2 ? 1 : 0)));
     args.out_f32 = out_kind == OUT_F32 ? 1 : 0;
     args.passes = passes;
     const int per_token = fp4 ? K / 32 : K / mfma_quarter_bytes<BITS>();  // staging tasks per token
@@ -121,9 +143,10 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
     const int grid_x = (N + rows_per_wg - 1) / rows_per_wg;
     const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
     const MfmaKernelFn fn = fp4 ? fp4_table<BITS>().fn[ri][variant]
-                                : (direct ? (nw == 8 ? mfma_direct8_table<BITS>().fn[ri][variant]
-                                                     : mfma_direct_table<BITS>().fn[ri][variant])
-                                          : mfma_table<BITS>().fn[ri][variant]);
+                                : (flex ? mfma_direct_flex_table<BITS>().fn[0][variant]
+                                   : direct ? (nw == 8 ? mfma_direct8_table<BITS>().fn[ri][variant]
+                                                       : mfma_direct_table<BITS>().fn[ri][variant])
+                                            : mfma_table<BITS>().fn[ri][variant]);
     hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(nw * 64, 1, 1), lds_for(ri, mt),
                        stream, args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
                        args.mt, args.ks_log2, args.out_f32, args.passes, args.div_magic);

@@ -317,14 +317,25 @@ __global__ void __launch_bounds__(kMfmaThreads) gemv_mfma_kernel
 // activations: the kernel is one memory round trip plus the K loop long.
 // ---------------------------------------------------------------------------
 // NW = waves per workgroup: four, or eight for long rows (K >= 4096), where a wave would
-// otherwise walk through several K tiles one memory round trip after the other.
+// otherwise walk through several K tiles one after the other.  NW = 0 is the form for tile
+// counts that are no power of two (K = 2560, 6144, 9728 ...): one row block per workgroup
+// and any number of waves up to twelve, each with its own K slice; the argument that
+// otherwise carries log2 of the split then carries the split itself.
+constexpr int kMfmaFlexMaxWaves = 12;
+
+template <int BITS, int R>
+__host__ __device__ inline size_t mfma_direct_lds_bytes_for(int nwaves) {
+    return (size_t)nwaves * mfma_wave_tile_bytes<BITS, R>() + (size_t)nwaves * R * 4 * 64 * 4;
+}
+
 template <int BITS, int R, int NW = 4>
 __host__ __device__ inline size_t mfma_direct_lds_bytes() {
-    return (size_t)NW * mfma_wave_tile_bytes<BITS, R>() + (size_t)NW * R * 4 * 64 * 4;
+    return mfma_direct_lds_bytes_for<BITS, R>(NW);
 }
 
 template <int BITS, int R, bool G32, bool SF16, int NW = 4>
-__global__ void __launch_bounds__(NW * 64) gemv_mfma_direct_kernel
+__global__ void __launch_bounds__(NW == 0 ? kMfmaFlexMaxWaves * 64 : NW * 64)
+gemv_mfma_direct_kernel
 (const int8_t *pA, const uint8_t *pB, void *pout, const float *ps, const uint16_t *pws, int pM,
  int pN, int pK, int pmt, int pks_log2, int pout_f32, int ppasses, uint32_t pdiv_magic) {
     // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
@@ -338,10 +349,12 @@ __global__ void __launch_bounds__(NW * 64) gemv_mfma_direct_kernel
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int ks = 1 << a.ks_log2;
-    const int kslice = wave & (ks - 1);
-    const int rw = wave >> a.ks_log2;
-    const int rws = NW >> a.ks_log2;
+    constexpr bool kFlex = NW == 0;
+    const int ks = kFlex ? a.ks_log2 : 1 << a.ks_log2;
+    const int nwaves = kFlex ? ks : NW;
+    const int kslice = kFlex ? wave : wave & (ks - 1);
+    const int rw = kFlex ? 0 : wave >> a.ks_log2;
+    const int rws = kFlex ? 1 : NW >> a.ks_log2;
     const int m0 = blockIdx.y * a.mt;
     const int mt = (M - m0) < a.mt ? (M - m0) : a.mt;
     const int pass_rows = rws * 16 * R;
@@ -349,11 +362,13 @@ __global__ void __launch_bounds__(NW * 64) gemv_mfma_direct_kernel
 
     unsigned char *tiles = smem;
     unsigned char *wt = tiles + (size_t)wave * mfma_wave_tile_bytes<BITS, R>();
-    float *red = reinterpret_cast<float *>(tiles + (size_t)NW * mfma_wave_tile_bytes<BITS, R>());
+    float *red =
+        reinterpret_cast<float *>(tiles + (size_t)nwaves * mfma_wave_tile_bytes<BITS, R>());
 
     const int ntiles = G / kMfmaGroupsPerTile;
-    const int t_begin = (int)(((long)ntiles * kslice) >> a.ks_log2);
-    const int t_end = (int)(((long)ntiles * (kslice + 1)) >> a.ks_log2);
+    const int t_begin = kFlex ? ntiles * kslice / ks : (int)(((long)ntiles * kslice) >> a.ks_log2);
+    const int t_end = kFlex ? ntiles * (kslice + 1) / ks
+                            : (int)(((long)ntiles * (kslice + 1)) >> a.ks_log2);
 
     const int ld_row = lane / MF::kLanesPerRow;
     const int ld_col = lane % MF::kLanesPerRow;
@@ -598,6 +613,19 @@ const MfmaTable<BITS> &mfma_direct_table() {
     return t;
 }
 
+// the form with one K slice per wave for any number of waves (one row tile per wave only)
+template <int BITS>
+const MfmaTable<BITS> &mfma_direct_flex_table() {
+    static const MfmaTable<BITS> t = [] {
+        MfmaTable<BITS> x{};
+        x.fn[0][0] = gemv_mfma_direct_kernel<BITS, 1, false, false, 0>;
+        x.fn[0][1] = gemv_mfma_direct_kernel<BITS, 1, false, true, 0>;
+        x.fn[0][2] = gemv_mfma_direct_kernel<BITS, 1, true, false, 0>;
+        return x;
+    }();
+    return t;
+}
+
 // the eight-wave form of the direct kernel
 template <int BITS>
 const MfmaTable<BITS> &mfma_direct8_table() {
@@ -619,12 +647,9 @@ const MfmaTable<BITS> &mfma_direct8_table() {
 
 template <int BITS>
 size_t mfma_direct_lds_for(int ri, int nw = 4) {
-    if (nw == 8)
-        return ri == 0 ? mfma_direct_lds_bytes<BITS, 1, 8>()
-                       : (ri == 1 ? mfma_direct_lds_bytes<BITS, 2, 8>()
-                                  : mfma_direct_lds_bytes<BITS, 4, 8>());
-    return ri == 0 ? mfma_direct_lds_bytes<BITS, 1>()
-                   : (ri == 1 ? mfma_direct_lds_bytes<BITS, 2>() : mfma_direct_lds_bytes<BITS, 4>());
+    return ri == 0 ? mfma_direct_lds_bytes_for<BITS, 1>(nw)
+                   : (ri == 1 ? mfma_direct_lds_bytes_for<BITS, 2>(nw)
+                              : mfma_direct_lds_bytes_for<BITS, 4>(nw));
 }
 
 template <int BITS>
@@ -635,12 +660,14 @@ MfmaTuning &mfma_tuning() {
 
 template <int BITS>
 int mfma_init_device(int max_lds) {
-    const MfmaTable<BITS> *tables[3] = {&mfma_table<BITS>(), &mfma_direct_table<BITS>(),
-                                        &mfma_direct8_table<BITS>()};
+    const MfmaTable<BITS> *tables[4] = {&mfma_table<BITS>(), &mfma_direct_table<BITS>(),
+                                        &mfma_direct8_table<BITS>(),
+                                        &mfma_direct_flex_table<BITS>()};
     for (const MfmaTable<BITS> *t : tables)
         for (int r = 0; r < 3; ++r)
             for (int v = 0; v < 3; ++v)
-                if (hipFuncSetAttribute(reinterpret_cast<const void *>(t->fn[r][v]),
+                if (t->fn[r][v] != nullptr &&
+                    hipFuncSetAttribute(reinterpret_cast<const void *>(t->fn[r][v]),
                                         hipFuncAttributeMaxDynamicSharedMemorySize,
                                         max_lds) != hipSuccess)
                     return 2;
