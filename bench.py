@@ -382,7 +382,7 @@ def main() -> int:
 
     # The other half of the headline metric: end-to-end decode tokens/s of the random-init
     # 1.7B-shaped model (configs[2]), AR and D8 hybrid, by the reference's timing contract.
-    decode = decode_bf16 = None
+    decode = decode_bf16 = decode_4b = None
     if not args.no_decode:
         del run, pool, graph
         torch.cuda.empty_cache()
@@ -393,6 +393,9 @@ def main() -> int:
         # the 83 MB packed head the reference's graphs use for a ternary backbone)
         decode_bf16 = run_decode_bench("1.7b", prompt_len=256, new_tokens=512, repeats=1,
                                        head_kind="bf16")
+        torch.cuda.empty_cache()
+        # configs[3]: the 4B-shaped model, 512-token prompt, 1024 new tokens
+        decode_4b = run_decode_bench("4b", prompt_len=512, new_tokens=1024, repeats=1)
 
     cpu = cpu_baseline(args.cpu_seconds) if args.cpu_seconds > 0 else None
 
@@ -414,6 +417,7 @@ def main() -> int:
             "lm_head_151936x2048": head,
             "decode_1p7b_d8": decode,
             "decode_1p7b_d8_bf16_lm_head": decode_bf16,
+            "decode_4b_d8": decode_4b,
         },
         "roofline": roofline,
         "cpu_baseline": cpu,
