@@ -438,6 +438,11 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
             if (low_waste && waves >= 2048) break;
         }
         lpr = best;
+        // 1-bit chunks carry 128 weights each, a long serial chain per lane: while the launch
+        // is short of waves anyway, more lanes per row (up to 32) until a lane has at most
+        // two chunks, idle lanes or not
+        if (BITS == 1 && ((long)N * lpr + 63) / 64 < 2048)
+            while (lpr < 32 && (C + lpr - 1) / lpr > 2) lpr *= 2;
     }
     g.lpr_log2 = ilog2(lpr);
     // loads per batch: the largest of 4, 2, 1 that wastes no load slot, 4 for long rows
