@@ -154,7 +154,8 @@ def test_q1_4b_shapes_full_size(oracle, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 2048), (9, 12288, 2048), (17, 2560, 9728),
-                                    (16, 19456, 2560), (12, 6144, 2560), (10, 2560, 4096)])
+                                    (16, 19456, 2560), (12, 6144, 2560), (10, 2560, 4096),
+                                    (9, 2048, 6144), (16, 4096, 2560), (9, 1024, 2560)])
 def test_t2_decode_widths_merged_shapes(oracle, M, N, K):
     """Merged decode shapes at the widths a D8 schedule replays (9..17)."""
     p = oracle.synth_problem(2, M, N, K, 2)
