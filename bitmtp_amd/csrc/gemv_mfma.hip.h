@@ -445,7 +445,10 @@ gemv_mfma_direct_kernel
     for (int rt = 0; rt < R; ++rt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[rt][r] = 0.0f;
-    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    // the offset-removal term straight from the matrix cores: -2 (T2) / -1 (Q1) in every slot
+    // of the B operand gives -2 * sum(a) / -sum(a) per token in the accumulator layout
+    constexpr int kNegs = BITS == 2 ? (int)0xFEFEFEFEu : (int)0xFFFFFFFFu;
+    const v4i negs = {kNegs, kNegs, kNegs, kNegs};
     const v4i zero = {0, 0, 0, 0};
 
     for (int pass = 0; pass < a.passes; ++pass) {
@@ -473,11 +476,8 @@ gemv_mfma_direct_kernel
                 }
                 const v4i va0 = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w};
                 const v4i va1 = {(int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
-                // sum of the group's activations per token, in the accumulator layout
-                v4i asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, ones, zero, 0, 0, 0);
-                asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, ones, asum, 0, 0, 0);
-                const v4i vcr = {mfma_corr<BITS>(asum[0]), mfma_corr<BITS>(asum[1]),
-                                 mfma_corr<BITS>(asum[2]), mfma_corr<BITS>(asum[3])};
+                v4i vcr = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, negs, zero, 0, 0, 0);
+                vcr = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, negs, vcr, 0, 0, 0);
 #pragma unroll
                 for (int rt = 0; rt < R; ++rt) {
                     const unsigned char *src = wt + (rt * 16 + op_row) * MF::kPitch;
