@@ -31,8 +31,8 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by a 256 MiB copy), from the
 # two rocprofv3 --pmc runs summarised under profiles/: mean over the seven launches of a
 # width.  Not measured live.
-MEASURED_TRAFFIC_BYTES = {1: (1971.2 + 6.9) * 1024, 4: (2034.7 + 22.9) * 1024,
-                          8: (2118.5 + 45.7) * 1024}
+MEASURED_TRAFFIC_BYTES = {1: (1971.3 + 6.9) * 1024, 4: (2031.1 + 22.9) * 1024,
+                          8: (2115.2 + 45.7) * 1024}
 WIDTHS = (1, 4, 8)
 # name, N, K  (Qwen3-1.7B: hidden 2048, 16 q / 8 kv heads x 128, ffn 6144)
 PROJECTIONS = (
