@@ -162,6 +162,16 @@ def test_t2_decode_widths_merged_shapes(oracle, M, N, K):
     check_problem(oracle, p, 2, "t2-merged")
 
 
+@pytest.mark.parametrize("bits", [2, 1])
+@pytest.mark.parametrize("M,N,K", [(1, 2049, 2048), (2, 4100, 2048), (1, 2050, 6144),
+                                    (9, 2050, 6144), (9, 4090, 2560), (16, 1030, 9728)])
+def test_ragged_rows_at_layer_size(oracle, bits, M, N, K):
+    """Row counts that are no multiple of a workgroup's rows, at sizes where the launcher
+    picks its eight-wave and one-slice-per-wave geometries."""
+    p = oracle.synth_problem(77 + M + N, M, N, K, bits)
+    check_problem(oracle, p, bits, "ragged")
+
+
 def test_t2_head_shape(oracle):
     """The packed lm_head: N = 151936, width D+1 = 9."""
     p = oracle.synth_problem(3, 9, 151936, 2048, 2)
