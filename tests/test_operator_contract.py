@@ -67,6 +67,20 @@ def test_generic_mode_accepts_every_aligned_shape():
             contracts.require_kernel_shape("t2g128", m, n, k)
 
 
+def test_shapes_past_the_launcher_limits_raise_before_the_native_call():
+    """The void drop-in symbol cannot report an error, so the wrapper must refuse what the
+    launcher would refuse: more than 2^30 output elements, rows longer than 65536."""
+    assert contracts.supports_kernel_shape("t2g128", 7067, 151936, 2048)       # just below 2^30
+    assert not contracts.supports_kernel_shape("t2g128", 7068, 151936, 2048)
+    assert not contracts.supports_kernel_shape("q1", 1, 8, 65536 + 128)
+    a = torch.empty(7068, 2048, dtype=torch.int8, device="meta")
+    b = torch.empty(151936, 512, dtype=torch.int8, device="meta")
+    s = torch.empty(7068, 1, dtype=torch.float32, device="meta")
+    ws = torch.empty(151936, 16, dtype=torch.bfloat16, device="meta")
+    with pytest.raises(RuntimeError, match="unsupported t2g128 kernel shape"):
+        ops.t2g128_int8xint2_linear(a, b, s, ws)
+
+
 @pytest.mark.parametrize("fn,bits,kind", [(ops.t2g128_int8xint2_linear, 2, "t2g128"),
                                           (ops.q1g128_int8xint1_linear, 1, "q1")])
 def test_validation_messages(fn, bits, kind, monkeypatch):
