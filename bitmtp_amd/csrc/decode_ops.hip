@@ -1436,6 +1436,44 @@ extern "C" int bonsai_draft_chain_ws(const void *logits, int rows, int ld, int v
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 
+// ---------------------------------------------------------------------------
+// The split draft chain for callers that cannot allocate: the partial statistics go through
+// a library-owned device array instead of a caller-supplied workspace.  The array's name is
+// only a host-side handle; its device address is looked up once per device and kept.
+// ---------------------------------------------------------------------------
+constexpr int kStaticScratchFloats = BONSAI_MAX_WIDTH * kDraftSplits * 4;  // 16 KiB
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+static float *g_static_scratch[kMaxDevices];  // device address of `scratch`, per device
+
+extern "C" int bonsai_draft_chain_static(const void *logits, int rows, int ld, int vocab,
+                                         float threshold, int32_t *tokens, float *conf,
+                                         int32_t *accept, void *stream) {
+    if (!logits || !tokens || !conf || !accept) return BONSAI_DECODE_ERR_ARG;
+    // rows beyond what the static array holds are refused, never truncated
+    if (rows < 1 || rows > BONSAI_MAX_WIDTH || vocab < 1 || ld < vocab || ld % 8 != 0)
+        return BONSAI_DECODE_ERR_ARG;
+    if ((size_t)rows * kDraftSplits * 4 > (size_t)kStaticScratchFloats) return BONSAI_DECODE_ERR_ARG;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
+    if (g_static_scratch[dev] == nullptr) {
+        float *ptr = nullptr;
+        if (hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess ||
+            ptr == nullptr)
+            return BONSAI_DECODE_ERR_LAUNCH;
+        g_static_scratch[dev] = ptr;
+    }
+    float *ws = g_static_scratch[dev];
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // every slot the merge reads is written by the split pass of the same call: nothing to clear
+    hipLaunchKernelGGL(draft_rows_split_kernel, dim3(rows * kDraftSplits), dim3(kDraftSplitThreads), 0,
+                       st, static_cast<const uint16_t *>(logits), ld, vocab, kDraftSplits, ws);
+    if (hipGetLastError() != hipSuccess) return BONSAI_DECODE_ERR_LAUNCH;
+    hipLaunchKernelGGL(draft_merge_accept_kernel, dim3(1), dim3(1024), 0, st,
+                       static_cast<const float *>(ws), rows, kDraftSplits, threshold, tokens, conf,
+                       accept);
+    return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
 extern "C" int bonsai_bf16_linear(const void *x, const void *w, void *out, int M, int N, int K,
                                   void *stream) {
     if (!x || !w || !out) return BONSAI_DECODE_ERR_ARG;

@@ -119,6 +119,18 @@ int bonsai_draft_chain_ws(const void *logits, int rows, int ld, int vocab, float
                           int32_t *tokens, float *conf, int32_t *accept, void *scratch,
                           void *stream);
 
+/* The split chain for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same kernels and outputs as bonsai_draft_chain_ws, but the partial statistics go
+ * through a 16 KiB device array owned by the library (one copy per GPU, held until the
+ * process ends) instead of a caller workspace; the call allocates and frees nothing.
+ * rows <= BONSAI_MAX_WIDTH, larger inputs are refused with BONSAI_DECODE_ERR_ARG.  All calls
+ * on one GPU share that array: calls that overlap in time on one GPU (different streams) race.
+ * The first call on a device looks the array's address up; make that call outside stream
+ * capture. */
+int bonsai_draft_chain_static(const void *logits, int rows, int ld, int vocab, float threshold,
+                              int32_t *tokens, float *conf, int32_t *accept, void *stream);
+
 /* bf16 output projection of a sign-weight (Q1) backbone, whose graphs keep the tied lm_head
  * in bf16: logits = F.linear(h, W) (`_lm_head`, precision "bf16",
  * src/bonsai_sft/gpu/model.py:1296; chosen in src/bonsai_sft/gpu/fast_runtime.py:175-178).
