@@ -16,6 +16,7 @@
 
 #include "gemv_fp4.hip.h"
 #include "gemv_mfma.hip.h"
+#include "gemv_mx.hip.h"
 #include "packed_gemv.hip.h"
 
 namespace bonsai {
@@ -36,6 +37,13 @@ int init_all_kernels() {
         if (rc2 != 0) return rc2;
         const int rc3 = fp4_init_device<BITS>(st.lds_limit[dev]);
         if (rc3 != 0) return rc3;
+        const int rc4 = mx_init_device<BITS>(st.lds_limit[dev]);
+        if (rc4 != 0) return rc4;
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            cus <= 0)
+            return 2;
+        st.n_cus[dev] = cus;
         st.mfma_ready[dev] = true;
     }
     return 0;
@@ -153,6 +161,31 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
+// One problem through the grouped kernel (token tiles of at most 16 as separate descriptors).
+// Returns -1 when it does not fit.
+template <int BITS>
+int launch_grouped_mx_only(const GemvProblem &q, int out_kind, int scale_kind, int lds_limit,
+                           int n_cus, hipStream_t stream) {
+    // (the staged activations are chunked along K, so any block of up to 16 tokens fits in LDS)
+    const int cap = q.M < kMfmaTokens ? q.M : kMfmaTokens;
+    const int ntt = (q.M + cap - 1) / cap;
+    if (ntt > kMxMaxDesc) return -1;
+    const int mt = (q.M + ntt - 1) / ntt;
+    const size_t out_elt = out_kind == OUT_BF16 ? 2 : 4;
+    GemvProblem batch[kMxMaxDesc];
+    int nb = 0;
+    for (int m0 = 0; m0 < q.M; m0 += mt) {
+        GemvProblem sub = q;
+        sub.M = (q.M - m0) < mt ? (q.M - m0) : mt;
+        sub.A = q.A + (size_t)m0 * q.K;
+        sub.s = q.s == nullptr ? nullptr : q.s + m0;
+        const size_t per_tok = out_kind == OUT_G32 ? (size_t)q.N * (q.K / kGroup) : (size_t)q.N;
+        sub.out = static_cast<unsigned char *>(q.out) + (size_t)m0 * per_tok * out_elt;
+        batch[nb++] = sub;
+    }
+    return launch_mx<BITS>(batch, nb, out_kind, scale_kind, lds_limit, n_cus, stream);
+}
+
 template <int BITS>
 int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
                 int M, int N, int K, int out_kind, int scale_kind, hipStream_t stream) {
@@ -174,6 +207,15 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     const MfmaTuning &mtu = mfma_tuning<BITS>();
     const int min_width = mtu.min_width > 0 ? mtu.min_width
                                             : (N >= kLongMatrixRows ? 2 : kDefaultMfmaMinWidth);
+    if (mtu.engine == 4 && M >= min_width) {
+        // the grouped kernel with a single descriptor
+        const GemvProblem q{A, B, out, s, ws, M, N, K};
+        if (mx_problem_ok(q, out_kind == OUT_G32)) {
+            const int rc = launch_grouped_mx_only<BITS>(q, out_kind, scale_kind, lds_limit, st.n_cus[dev],
+                                                        stream);
+            if (rc >= 0) return rc;
+        }
+    }
     if (M >= min_width && mfma_shape_ok(B, out_kind == OUT_G32 ? nullptr : ws, K)) {
         int rc = -1;
         // operand-loaded activations win up to about 16k rows, staged ones above (measured)
@@ -188,6 +230,73 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     }
     return launch_gemv_dot4<BITS>(A, B, out, s, ws, M, N, K, out_kind, scale_kind, lds_limit,
                                   stream);
+}
+
+// Several GEMVs in one call (descriptors in host memory, read before the call returns).
+// Problems the grouped kernel takes (K % 512 == 0, aligned operands) share launches of up to
+// kMxMaxDesc descriptors each, blocks wider than 16 tokens as several token tiles; the rest
+// go through launch_gemv one by one.  The arithmetic of every problem is that of the
+// single-GEMV entry points.
+template <int BITS>
+int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_kind,
+                   hipStream_t stream) {
+    if (probs == nullptr || count < 1) return 1;
+    if (out_kind < 0 || out_kind > 2 || scale_kind < 0 || scale_kind > 1) return 1;
+    for (int i = 0; i < count; ++i) {
+        const GemvProblem &q = probs[i];
+        if (q.A == nullptr || q.B == nullptr || q.out == nullptr) return 1;
+        if (out_kind != OUT_G32 && (q.s == nullptr || q.ws == nullptr)) return 1;
+        if (q.M < 1 || q.N < 1 || q.K < kGroup || q.K % kGroup != 0) return 1;
+        if ((long)q.M * q.N > 0x7fffffffL / 2) return 1;
+    }
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 2;
+    LibState<BITS> &st = lib_state<BITS>();
+    if (st.lds_limit[dev] == 0 || !st.mfma_ready[dev]) {
+        const int rc = init_all_kernels<BITS>();
+        if (rc != 0) return rc;
+    }
+    const int lds_limit = st.lds_limit[dev];
+    const MxTuning &tu = mx_tuning<BITS>();
+    const int min_width = tu.min_width > 0 ? tu.min_width : 1;
+
+    GemvProblem batch[kMxMaxDesc];
+    int nb = 0;
+    auto flush = [&]() -> int {
+        if (nb == 0) return 0;
+        const int rc = launch_mx<BITS>(batch, nb, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
+        nb = 0;
+        return rc;
+    };
+    const size_t out_elt = out_kind == OUT_BF16 ? 2 : 4;
+    for (int i = 0; i < count; ++i) {
+        const GemvProblem &q = probs[i];
+        // token tiles of at most 16 (the staged activations are chunked along K: they always fit)
+        const int cap = q.M < kMfmaTokens ? q.M : kMfmaTokens;
+        if (q.M < min_width || !mx_problem_ok(q, out_kind == OUT_G32)) {
+            const int rc = launch_gemv<BITS>(q.A, q.B, q.out, q.s, q.ws, q.M, q.N, q.K, out_kind,
+                                             scale_kind, stream);
+            if (rc != 0) return rc;
+            continue;
+        }
+        const int ntt = (q.M + cap - 1) / cap;
+        const int mt = (q.M + ntt - 1) / ntt;
+        for (int m0 = 0; m0 < q.M; m0 += mt) {
+            GemvProblem sub = q;
+            sub.M = (q.M - m0) < mt ? (q.M - m0) : mt;
+            sub.A = q.A + (size_t)m0 * q.K;
+            sub.s = q.s == nullptr ? nullptr : q.s + m0;
+            const size_t per_tok = out_kind == OUT_G32 ? (size_t)q.N * (q.K / kGroup) : (size_t)q.N;
+            sub.out = static_cast<unsigned char *>(q.out) + (size_t)m0 * per_tok * out_elt;
+            batch[nb++] = sub;
+            if (nb == kMxMaxDesc) {
+                const int rc = flush();
+                if (rc != 0) return rc < 0 ? 2 : rc;
+            }
+        }
+    }
+    const int rc = flush();
+    return rc < 0 ? 2 : rc;
 }
 
 }  // namespace bonsai

@@ -347,6 +347,7 @@ struct LibState {
     Tuning tuning;
     int lds_limit[kMaxDevices] = {};  // 0 = device not initialised yet
     bool mfma_ready[kMaxDevices] = {};
+    int n_cus[kMaxDevices] = {};
 };
 
 template <int BITS>

@@ -27,6 +27,23 @@ void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passe
     t.engine = engine;
 }
 
+int t2g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, int scale_kind,
+                        void *stream) {
+    if (descs == nullptr || count < 1 || count > BONSAI_GROUPED_MAX) return BONSAI_ERR_ARG;
+    GemvProblem probs[BONSAI_GROUPED_MAX];
+    for (int i = 0; i < count; ++i)
+        probs[i] = GemvProblem{descs[i].A, descs[i].B, descs[i].out, descs[i].s, descs[i].ws,
+                               descs[i].M, descs[i].N, descs[i].K};
+    return launch_grouped<2>(probs, count, out_kind, scale_kind, static_cast<hipStream_t>(stream));
+}
+
+void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width) {
+    MxTuning &t = mx_tuning<2>();
+    t.row_tiles = row_tiles;
+    t.max_wgs = max_wgs;
+    t.min_width = min_width;
+}
+
 int t2g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
                    int M, int N, int K, int out_kind, int scale_kind, void *stream) {
     return launch_gemv<2>(A, B, out, s, ws, M, N, K, out_kind, scale_kind,

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from typing import Optional, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -35,6 +35,19 @@ _GEMV_EX_ARGTYPES = [
     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
     ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
 ]
+
+
+class GemvDesc(ctypes.Structure):
+    """``bonsai_gemv_desc`` of include/bonsai_gemv.h: one GEMV of a grouped call."""
+    _fields_ = [("A", ctypes.c_void_p), ("B", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("s", ctypes.c_void_p), ("ws", ctypes.c_void_p),
+                ("M", ctypes.c_int32), ("N", ctypes.c_int32), ("K", ctypes.c_int32),
+                ("reserved", ctypes.c_int32)]
+
+
+GROUPED_MAX = 64
+_GROUPED_ARGTYPES = [ctypes.POINTER(GemvDesc), ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                     ctypes.c_void_p]
 
 
 def _open(relpath: str) -> ctypes.CDLL:
@@ -72,6 +85,10 @@ def load_t2_kernel() -> None:
     lib.t2g128_set_tuning.restype = None
     lib.t2g128_set_mfma_tuning.argtypes = [ctypes.c_int] * 5
     lib.t2g128_set_mfma_tuning.restype = None
+    lib.t2g128_gemv_grouped.argtypes = _GROUPED_ARGTYPES
+    lib.t2g128_gemv_grouped.restype = ctypes.c_int
+    lib.t2g128_set_grouped_tuning.argtypes = [ctypes.c_int] * 3
+    lib.t2g128_set_grouped_tuning.restype = None
     _t2_lib = lib
 
 
@@ -94,6 +111,10 @@ def load_q1_kernel() -> None:
     lib.q1g128_set_tuning.restype = None
     lib.q1g128_set_mfma_tuning.argtypes = [ctypes.c_int] * 5
     lib.q1g128_set_mfma_tuning.restype = None
+    lib.q1g128_gemv_grouped.argtypes = _GROUPED_ARGTYPES
+    lib.q1g128_gemv_grouped.restype = ctypes.c_int
+    lib.q1g128_set_grouped_tuning.argtypes = [ctypes.c_int] * 3
+    lib.q1g128_set_grouped_tuning.restype = None
     _q1_lib = lib
 
 
@@ -287,6 +308,66 @@ def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[tor
     if rc != 0:
         raise RuntimeError(f"{kind}: native launch failed with status {rc} (M={m}, N={n}, K={k})")
     return out
+
+
+def packed_gemv_grouped(problems: Sequence[Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor],
+                                                 Optional[torch.Tensor]]],
+                        *, bits: int, out_kind: int = OUT_BF16,
+                        outs: Optional[Sequence[torch.Tensor]] = None) -> List[torch.Tensor]:
+    """Several independent GEMVs ``(a_int8 [M,K], b_packed, s, ws)`` in one native call
+    (``*_gemv_grouped``): one launch walks the row tiles of all of them.  Widths, row counts
+    and K may differ between the problems; every result is what ``packed_gemv_ex`` gives for
+    that problem alone.  ``outs`` supplies preallocated outputs (so that a captured graph
+    allocates nothing); otherwise fresh tensors are returned."""
+    if bits not in (1, 2):
+        raise ValueError("bits must be 1 (Q1) or 2 (T2)")
+    if not 1 <= len(problems) <= GROUPED_MAX:
+        raise ValueError(f"a grouped call takes 1..{GROUPED_MAX} problems")
+    if out_kind not in (OUT_BF16, OUT_F32, OUT_G32):
+        raise ValueError("bad out_kind")
+    if outs is not None and len(outs) != len(problems):
+        raise ValueError("one output per problem")
+    kind = "t2g128" if bits == 2 else "q1"
+    descs = (GemvDesc * len(problems))()
+    results: List[torch.Tensor] = []
+    dev = problems[0][0].device
+    scale_kinds = set()
+    for i, (a, b, s, ws) in enumerate(problems):
+        if a.dim() != 2:
+            raise ValueError(f"{kind}: expected rank-2 activation")
+        if out_kind == OUT_G32:
+            if b.dim() != 2:
+                raise ValueError(f"{kind}: expected rank-2 weight")
+            require_kernel_shape(kind, a.shape[0], b.shape[0], b.shape[1] * (8 // bits))
+        else:
+            _validate_packed_inputs(a, b, s, ws, kind=kind, bits=bits, activation_dtype=torch.int8,
+                                    scale_dtypes=(torch.bfloat16, torch.float16))
+            scale_kinds.add(SCALE_F16 if ws.dtype == torch.float16 else SCALE_BF16)
+        if a.device != dev:
+            raise RuntimeError(f"{kind}: all problems of a grouped call must share one CUDA device")
+        m, n, k = a.shape[0], b.shape[0], b.shape[1] * (8 // bits)
+        shape = (m, n, k // 128) if out_kind == OUT_G32 else (m, n)
+        dtype = {OUT_BF16: torch.bfloat16, OUT_F32: torch.float32, OUT_G32: torch.int32}[out_kind]
+        if outs is None:
+            out = torch.empty(*shape, dtype=dtype, device=dev)
+        else:
+            out = outs[i]
+            if tuple(out.shape) != shape or out.dtype != dtype or out.device != dev or \
+                    not out.is_contiguous():
+                raise RuntimeError(f"{kind}: output {i} must be a contiguous {dtype} tensor {shape}")
+        results.append(out)
+        descs[i] = GemvDesc(a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                            None if s is None else s.data_ptr(),
+                            None if ws is None else ws.data_ptr(), m, n, k, 0)
+    if len(scale_kinds) > 1:
+        raise RuntimeError(f"{kind}: the scales of a grouped call must share one dtype")
+    scale_kind = scale_kinds.pop() if scale_kinds else SCALE_BF16
+    fn = t2_lib().t2g128_gemv_grouped if bits == 2 else q1_lib().q1g128_gemv_grouped
+    with torch.cuda.device(dev):
+        rc = fn(descs, len(problems), out_kind, scale_kind, _stream(dev))
+    if rc != 0:
+        raise RuntimeError(f"{kind}: grouped native launch failed with status {rc}")
+    return results
 
 
 def quant_input(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -85,6 +85,32 @@ int t2g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s,
 int q1g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
                    int M, int N, int K, int out_kind, int scale_kind, void *stream);
 
+/* ---- several GEMVs in one launch ------------------------------------------ */
+/* No counterpart in the reference, which launches one kernel per projection
+ * (src/bonsai_sft/gpu/model.py:977,1006,1058,1062 through t2g128_kernels.cu:94-100).  A
+ * layer-sized matrix (0.5-3.3 MB) is far too small to amortise a kernel launch, so GEMVs
+ * that do not depend on each other -- q|k|v, gate|up, or a whole layer in a throughput
+ * measurement -- can be handed over together: one grid walks the row tiles of all of them.
+ * Every descriptor is an independent GEMV with the operands and the result of the
+ * single-GEMV entry points above (same arithmetic: exact int32 group sums, fp32 scale
+ * accumulation, division by s[m], bf16 RNE); widths, row counts and K may differ between
+ * descriptors.  `descs` is HOST memory and is read before the call returns; the pointers
+ * inside are device pointers.  out_kind / scale_kind apply to all descriptors. */
+typedef struct bonsai_gemv_desc {
+    const int8_t *A;   /* int8 [M, K] */
+    const uint8_t *B;  /* packed weights [N, K/4] (T2) or [N, K/8] (Q1) */
+    void *out;         /* bf16 / fp32 [M, N] or int32 [M, N, K/128], see out_kind */
+    const float *s;    /* fp32 [M] */
+    const void *ws;    /* 16-bit [N, K/128] */
+    int32_t M, N, K;
+    int32_t reserved;  /* set to 0 */
+} bonsai_gemv_desc;
+#define BONSAI_GROUPED_MAX 64 /* descriptors per call */
+int t2g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, int scale_kind,
+                        void *stream);
+int q1g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, int scale_kind,
+                        void *stream);
+
 /* One-time set-up for the current device (raises the kernels' dynamic-LDS
  * limit).  Called implicitly by the first launch; call it explicitly before
  * capturing a graph if the first launch would otherwise happen under capture.
@@ -106,6 +132,12 @@ void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
  * otherwise int8 MFMA).  Zero = built-in choice. */
 void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
 void q1g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
+
+/* Development hook of the grouped kernel: 16-row tiles per wave (1 or 2), cap on the
+ * workgroups of one launch, smallest width sent to it.  Zero = built-in choice.  Process-wide,
+ * not thread-safe. */
+void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
+void q1g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
 
 /* ---- activation quantisation (libbonsai_actq.so) ------------------------- */
 /* Per-token symmetric INT8 quantisation, the native form of `quant_input`

@@ -1,0 +1,172 @@
+"""GPU parity of the grouped GEMV entry points (`t2g128_gemv_grouped`, `q1g128_gemv_grouped`)
+against the CPU oracle, through the C ABI: every descriptor of a call is checked as a GEMV of
+its own -- int32 group sums bit-exact, fp32 value within rtol 1e-3 / atol 1e-3, bf16 output the
+oracle's or the neighbouring representable value, and equal to the RNE rounding of the fp32
+value the same call returns.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import bf16_bits, bf16_ordinal, to_dev
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-3
+ATOL = 1e-3
+
+LAYER_17B = [(2048, 2048), (1024, 2048), (1024, 2048), (2048, 2048), (6144, 2048), (6144, 2048),
+             (2048, 6144)]
+LAYER_4B = [(4096, 2560), (1024, 2560), (1024, 2560), (2560, 4096), (9728, 2560), (9728, 2560),
+            (2560, 9728)]
+
+
+def check_group(O, probs, bits, label):
+    import bitmtp_amd as ops
+    dev = [to_dev(p) for p in probs]
+    shapes = [(p["A"].shape[0], p["B"].shape[0], p["A"].shape[1]) for p in probs]
+    print(f"[case] grouped {label} bits={bits} (M,N,K)={shapes}", flush=True)
+    G = ops.packed_gemv_grouped([(A, B, None, None) for A, B, s, ws in dev], bits=bits,
+                                out_kind=ops.OUT_G32)
+    y32 = ops.packed_gemv_grouped(dev, bits=bits, out_kind=ops.OUT_F32)
+    y16 = ops.packed_gemv_grouped(dev, bits=bits, out_kind=ops.OUT_BF16)
+    torch.cuda.synchronize()
+    for i, p in enumerate(probs):
+        G_ref = O.c_group_sums(p["A"], p["B"], bits)
+        y32_ref, y16_ref = O.c_gemv(p["A"], p["B"], p["s"], p["ws"], bits)
+        assert np.array_equal(G[i].cpu().numpy(), G_ref), f"{label}[{i}]: int32 group sums differ"
+        got = y32[i].cpu().numpy()
+        err = np.abs(got - y32_ref)
+        assert np.all(err <= ATOL + RTOL * np.abs(y32_ref)), f"{label}[{i}]: fp32 max err {err.max()}"
+        d = np.abs(bf16_ordinal(bf16_bits(y16[i])) - bf16_ordinal(y16_ref))
+        assert d.max() <= 1, f"{label}[{i}]: bf16 output more than one representable value away"
+        assert np.array_equal(bf16_bits(y16[i]), O.f32_to_bf16_bits(got)), f"{label}[{i}]: bf16 != rne(fp32)"
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 9, 17])
+def test_t2_17b_layer_in_one_call(oracle, M):
+    """All seven projections of the 1.7B-shaped layer (K = 2048 and 6144 mixed) in one call."""
+    probs = [oracle.synth_problem(10 * M + i, M, n, k, 2) for i, (n, k) in enumerate(LAYER_17B)]
+    check_group(oracle, probs, 2, f"1.7B layer M={M}")
+
+
+@pytest.mark.parametrize("M", [1, 8, 16])
+def test_t2_4b_layer_in_one_call(oracle, M):
+    """The 4B-shaped layer: K in {2560, 4096, 9728} (5, 8 and 19 K tiles over four waves)."""
+    probs = [oracle.synth_problem(20 * M + i, M, n, k, 2) for i, (n, k) in enumerate(LAYER_4B)]
+    check_group(oracle, probs, 2, f"4B layer M={M}")
+
+
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_q1_4b_set_in_one_call(oracle, M):
+    shapes = [(1024, 2560), (2560, 2560), (9728, 2560), (1024, 9728), (2560, 9728)]
+    probs = [oracle.synth_problem(30 * M + i, M, n, k, 1) for i, (n, k) in enumerate(shapes)]
+    check_group(oracle, probs, 1, f"Q1 4B set M={M}")
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+def test_mixed_widths_ragged_rows_and_odd_k(oracle, bits):
+    """Different M, N, K per descriptor; row counts that are no multiple of 16; K values the
+    grouped kernel does not take (below 2048 or no multiple of 512: they run through the
+    single-GEMV path inside the same call); blocks wider than 16 tokens."""
+    shapes = [(1, 2049, 2048), (9, 17, 512), (17, 130, 1024), (4, 1, 2560), (8, 1030, 6144),
+              (2, 33, 384), (33, 9, 640), (16, 50, 9728), (5, 255, 1536), (3, 100, 128)]
+    probs = [oracle.synth_problem(400 + i, m, n, k, bits) for i, (m, n, k) in enumerate(shapes)]
+    check_group(oracle, probs, bits, "mixed")
+
+
+def test_more_descriptors_than_one_launch_holds(oracle):
+    """40 small problems: more than the 24 descriptors of one launch."""
+    rng = np.random.default_rng(5)
+    probs = []
+    for i in range(40):
+        m, n, k = int(rng.integers(1, 18)), int(rng.integers(1, 200)), 512 * int(rng.integers(4, 9))
+        probs.append(oracle.synth_problem(600 + i, m, n, k, 2))
+    check_group(oracle, probs, 2, "many")
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+@pytest.mark.parametrize("row_tiles,max_wgs", [(1, 0), (2, 0), (1, 7), (2, 5), (1, 16), (2, 64)])
+def test_grouped_geometries(oracle, bits, row_tiles, max_wgs):
+    """One or two row tiles per wave compute the same thing, also when a small cap on the
+    workgroups makes every workgroup stride over several row-block iterations (the path the
+    151936-row head takes), restaging its activation tiles as it goes."""
+    from bitmtp_amd import ops as O2
+    lib = O2.t2_lib() if bits == 2 else O2.q1_lib()
+    setter = lib.t2g128_set_grouped_tuning if bits == 2 else lib.q1g128_set_grouped_tuning
+    shapes = [(1, 300, 2048), (8, 77, 2560), (16, 200, 4096), (5, 129, 6144), (3, 64, 3072), (16, 40, 9728),
+              (9, 33, 2048)]
+    try:
+        setter(row_tiles, max_wgs, 0)
+        probs = [oracle.synth_problem(700 + 10 * row_tiles + i, m, n, k, bits)
+                 for i, (m, n, k) in enumerate(shapes)]
+        check_group(oracle, probs, bits, f"geom R={row_tiles} cap={max_wgs}")
+    finally:
+        setter(0, 0, 0)
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+def test_grouped_arbitrary_bytes_and_extreme_activations(oracle, bits):
+    rng = np.random.default_rng(9)
+    probs = []
+    for i, (M, N, K) in enumerate([(6, 96, 1536), (1, 40, 512)]):
+        p = oracle.synth_problem(800 + i, M, N, K, bits)
+        p["A"] = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+        p["A"][0, :] = -128
+        p["B"] = rng.integers(0, 256, size=p["B"].shape, dtype=np.uint8)
+        p["B"][0, :] = 0x00
+        p["B"][1, :] = 0xFF
+        probs.append(p)
+    check_group(oracle, probs, bits, "extreme")
+
+
+def test_grouped_head_and_single_descriptor(oracle):
+    """One descriptor is a valid group: the packed lm_head at width 9."""
+    check_group(oracle, [oracle.synth_problem(3, 9, 151936, 2048, 2)], 2, "head")
+
+
+def test_grouped_equals_single_calls_bit_for_bit_per_kernel(oracle):
+    """The grouped kernel through the single-GEMV entry point (engine 4) returns exactly what
+    the grouped call returns for the same problem: the result does not depend on what else
+    shares the launch."""
+    import bitmtp_amd as ops
+    from bitmtp_amd import ops as O2
+    probs = [oracle.synth_problem(900 + i, 8, n, k, 2) for i, (n, k) in enumerate(LAYER_17B[3:])]
+    dev = [to_dev(p) for p in probs]
+    grouped = ops.packed_gemv_grouped(dev, bits=2, out_kind=ops.OUT_F32)
+    lib = O2.t2_lib()
+    try:
+        lib.t2g128_set_mfma_tuning(1, 0, 0, 0, 4)
+        for i, (A, B, s, ws) in enumerate(dev):
+            alone = ops.packed_gemv_ex(A, B, s, ws, bits=2, out_kind=ops.OUT_F32)
+            assert torch.equal(alone, grouped[i])
+    finally:
+        lib.t2g128_set_mfma_tuning(0, 0, 0, 0, 0)
+
+
+def test_grouped_graph_replay_and_argument_errors(oracle):
+    import bitmtp_amd as ops
+    ops.init_kernels()
+    probs = [oracle.synth_problem(950 + i, 8, n, k, 2) for i, (n, k) in enumerate(LAYER_17B)]
+    dev = [to_dev(p) for p in probs]
+    eager = [t.clone() for t in ops.packed_gemv_grouped(dev, bits=2)]
+    outs = [torch.empty_like(t) for t in eager]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        ops.packed_gemv_grouped(dev, bits=2, outs=outs)
+    for rep in range(3):
+        for t in outs:
+            t.zero_()
+        _ = ops.packed_gemv_grouped(dev, bits=2)   # eager work between replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, eager):
+            assert torch.equal(a, b), f"replay {rep} differs"
+    with pytest.raises(ValueError):
+        ops.packed_gemv_grouped([], bits=2)
+    with pytest.raises(RuntimeError):
+        ops.packed_gemv_grouped(dev, bits=2, outs=[torch.empty(1, 1, device="cuda:0")] * len(dev))
+    A, B, s, ws = dev[0]
+    with pytest.raises(RuntimeError):
+        ops.packed_gemv_grouped([(A, B[:, :-32].contiguous(), s, ws)], bits=2)
