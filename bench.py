@@ -3,16 +3,23 @@
 
 Workload (BASELINE.json configs[1]): all seven linear projections of one
 Qwen3-1.7B-shaped decoder layer in T2-g128 -- q/o 2048x2048, k/v 1024x2048,
-gate/up 6144x2048, down 2048x6144 -- at widths 1, 4 and 8, through the drop-in
-C entry point ``t2g128_int8xint2_linear``.  One STEP is that set once: 3 widths x
-7 projections = 21 launches.  Every launch reads a different layer of a pool of
-distinct random layers larger than the 256 MB Infinity Cache, so the weights come
-from HBM, and the steps are replayed from one HIP graph so that the Python launch
-cost is outside the measurement, as in the reference's graph-replayed decode.
+gate/up 6144x2048, down 2048x6144 -- at widths 1, 4 and 8.  One STEP is that set
+once.  It is measured two ways:
+
+* grouped (the headline `value`): the seven projections of a width handed to
+  ``t2g128_gemv_grouped`` together, one launch per width, 3 launches per step;
+* drop-in: one launch per projection through ``t2g128_int8xint2_linear``, the
+  reference's own launch structure, 21 launches per step (``config.drop_in``).
+
+Every launch reads a different layer of a pool of distinct random layers larger than
+the 256 MB Infinity Cache, so the weights come from HBM; every timed graph walks at
+least 512 MB of distinct weights whatever --steps is; the steps are replayed from one
+HIP graph so that the Python launch cost is outside the measurement, as in the
+reference's graph-replayed decode.
 
 Prints ONE JSON line: the driver's fields (metric, value, unit, ...), `config` with the
-per-width, merged-shape, lm_head and end-to-end decode figures, `roofline` of the slowest
-layer kernel and `cpu_baseline`.
+per-width, drop-in, merged-shape, lm_head and end-to-end decode figures, `roofline` of the
+dominant kernel and `cpu_baseline`.
 """
 from __future__ import annotations
 
@@ -28,11 +35,22 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by a 256 MiB copy), from the
-# two rocprofv3 --pmc runs summarised under profiles/: mean over the seven launches of a
-# width.  Not measured live.
-MEASURED_TRAFFIC_BYTES = {1: (1971.3 + 6.9) * 1024, 4: (2031.1 + 22.9) * 1024,
-                          8: (2115.2 + 45.7) * 1024}
+MIN_DISTINCT_BYTES = 512 << 20   # every timed graph walks at least this much distinct weight data
+
+
+def measured_traffic(width: int):
+    """HBM bytes per launch of the grouped kernel at `width` (FETCH_SIZE + WRITE_SIZE of two
+    rocprofv3 --pmc runs, each scaled by a 256 MiB copy), read from profiles/traffic.json --
+    the file the counter summaries under profiles/ are condensed into; None when absent."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            table = json.load(f)
+        return table["grouped_t2_layer_1p7b"][str(width)]["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 WIDTHS = (1, 4, 8)
 # name, N, K  (Qwen3-1.7B: hidden 2048, 16 q / 8 kv heads x 128, ffn 6144)
 PROJECTIONS = (
@@ -102,6 +120,8 @@ class Runner:
         self.pool = pool
         self.acts = acts
         self.fn = ops_mod.t2_lib().t2g128_int8xint2_linear
+        self.grouped = ops_mod.t2_lib().t2g128_gemv_grouped
+        self.desc_type = ops_mod.GemvDesc
         self.outs = {(m, i): torch.empty(m, n, dtype=torch.bfloat16, device=dev)
                      for m in WIDTHS for i, (_, n, _) in enumerate(PROJECTIONS)}
         self.cursor = 0  # next pool layer
@@ -115,45 +135,34 @@ class Runner:
             self.fn(q.data_ptr(), packed.data_ptr(), self.outs[(m, i)].data_ptr(), s.data_ptr(),
                     scales.data_ptr(), m, n, k, stream_ptr)
 
-    def step(self, widths, stream_ptr):
-        for m in widths:
-            self.launch_layer(m, stream_ptr)
+    def launch_layer_grouped(self, m: int, stream_ptr):
+        """The seven projections of one layer in ONE launch (t2g128_gemv_grouped)."""
+        layer = self.pool[self.cursor % len(self.pool)]
+        self.cursor += 1
+        descs = (self.desc_type * len(PROJECTIONS))()
+        for i, (_, n, k) in enumerate(PROJECTIONS):
+            q, s = self.acts[(m, k)]
+            packed, scales = layer[i]
+            descs[i] = self.desc_type(q.data_ptr(), packed.data_ptr(), self.outs[(m, i)].data_ptr(),
+                                      s.data_ptr(), scales.data_ptr(), m, n, k, 0)
+        rc = self.grouped(descs, len(PROJECTIONS), 0, 0, stream_ptr)
+        if rc != 0:
+            raise RuntimeError(f"t2g128_gemv_grouped failed with status {rc}")
 
-    def capture(self, n_steps: int, widths):
+    def step(self, widths, stream_ptr, grouped=False):
+        for m in widths:
+            if grouped:
+                self.launch_layer_grouped(m, stream_ptr)
+            else:
+                self.launch_layer(m, stream_ptr)
+
+    def capture(self, n_steps: int, widths, grouped=False):
         torch = self.torch
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             for _ in range(n_steps):
-                self.step(widths, sp)
-        return g
-
-    def capture_concurrent(self, n_steps: int, widths, n_streams: int):
-        """The same launches spread round-robin over `n_streams` forked streams inside one
-        graph: the projections of a step do not depend on each other, so this shows what the
-        kernels stream when a launch does not wait for its predecessor."""
-        torch = self.torch
-        g = torch.cuda.CUDAGraph()
-        sides = [torch.cuda.Stream() for _ in range(n_streams)]
-        with torch.cuda.graph(g):
-            main = torch.cuda.current_stream()
-            for s in sides:
-                s.wait_stream(main)
-            k = 0
-            for _ in range(n_steps):
-                for m in widths:
-                    layer = self.pool[self.cursor % len(self.pool)]
-                    self.cursor += 1
-                    for i, (_, n, kk) in enumerate(PROJECTIONS):
-                        q, s_ = self.acts[(m, kk)]
-                        packed, scales = layer[i]
-                        st = sides[k % n_streams]
-                        k += 1
-                        self.fn(q.data_ptr(), packed.data_ptr(), self.outs[(m, i)].data_ptr(),
-                                s_.data_ptr(), scales.data_ptr(), m, n, kk,
-                                ctypes.c_void_p(st.cuda_stream))
-            for s in sides:
-                main.wait_stream(s)
+                self.step(widths, sp, grouped)
         return g
 
     def time_graph(self, g) -> float:
@@ -165,6 +174,11 @@ class Runner:
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3  # seconds
+
+    def time_stats(self, g, replays: int = 5):
+        """(best, median) seconds over `replays` timed replays of one graph."""
+        ts = sorted(self.time_graph(g) for _ in range(replays))
+        return ts[0], ts[len(ts) // 2]
 
 
 def cpu_baseline(budget_s: float):
@@ -225,8 +239,8 @@ def cpu_baseline(budget_s: float):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=192)
-    ap.add_argument("--warmup", type=int, default=24)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=48, help="distinct layers in the weight pool")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--no-decode", action="store_true",
@@ -255,42 +269,77 @@ def main() -> int:
     acts = make_activations(torch, ops, seed=1, dev=dev)
     run = Runner(torch, ops_mod, pool, acts, dev)
 
-    # warm-up: eager steps (loads code objects), then one untimed replay of the timed graph
+    # warm-up: eager steps of both launch structures (loads code objects)
     sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     for _ in range(max(args.warmup, 1)):
-        run.step(WIDTHS, sp)
+        run.step(WIDTHS, sp, grouped=True)
+    run.step(WIDTHS, sp, grouped=False)
     torch.cuda.synchronize()
-
-    run.cursor = 0
-    graph = run.capture(args.steps, WIDTHS)
-    graph.replay()
-    torch.cuda.synchronize()
-    elapsed = min(run.time_graph(graph) for _ in range(3))
 
     step_bytes = len(WIDTHS) * LAYER_BYTES
-    gbps = step_bytes * args.steps / elapsed / 1e9
-    ms_per_step = elapsed / args.steps * 1e3
+    # steps per timed graph: the K asked for, and enough of them to walk >= 512 MB of distinct
+    # weights (a graph of n steps touches n * 3 layers; the pool is cycled, so also cap at it)
+    def graph_steps(bytes_per_step):
+        need = -(-MIN_DISTINCT_BYTES // bytes_per_step)
+        return max(args.steps, need)
 
-    # per-width: the same stream with one width only (7 launches per step)
-    per_width = {}
-    for m in WIDTHS:
-        run.cursor = 0
-        g = run.capture(args.steps, (m,))
-        g.replay()
-        torch.cuda.synchronize()
-        t = min(run.time_graph(g) for _ in range(3))
-        launches = args.steps * len(PROJECTIONS)
-        per_width[m] = {
-            "gbps": round(LAYER_BYTES * args.steps / t / 1e9, 1),
-            "pct_hbm_peak": round(LAYER_BYTES * args.steps / t / 1e9 / HBM_PEAK_GBPS * 100, 2),
-            "us_per_layer": round(t / args.steps * 1e6, 3),
-            "us_per_launch": round(t / launches * 1e6, 3),
-        }
-        del g
+    # ---- headline: grouped, one launch per width, exactly args.steps steps timed; when that
+    # is too few to leave the Infinity Cache behind, the graph holds more steps and the time
+    # of args.steps of them is reported
+    n_g = graph_steps(step_bytes)
+    run.cursor = 0
+    graph = run.capture(n_g, WIDTHS, grouped=True)
+    graph.replay()
+    torch.cuda.synchronize()
+    best, med = run.time_stats(graph)
+    elapsed = best * args.steps / n_g
+    gbps = step_bytes * n_g / best / 1e9
+    ms_per_step = best / n_g * 1e3
+    headline_median_gbps = step_bytes * n_g / med / 1e9
+    del graph
+
+    def width_table(grouped: bool):
+        table = {}
+        launches_per_layer = 1 if grouped else len(PROJECTIONS)
+        n = graph_steps(LAYER_BYTES)
+        for m in WIDTHS:
+            run.cursor = 0
+            g = run.capture(n, (m,), grouped=grouped)
+            g.replay()
+            torch.cuda.synchronize()
+            t, t_med = run.time_stats(g)
+            table[m] = {
+                "gbps": round(LAYER_BYTES * n / t / 1e9, 1),
+                "pct_hbm_peak": round(LAYER_BYTES * n / t / 1e9 / HBM_PEAK_GBPS * 100, 2),
+                "median_pct_hbm_peak": round(LAYER_BYTES * n / t_med / 1e9 / HBM_PEAK_GBPS * 100, 2),
+                "us_per_layer": round(t / n * 1e6, 3),
+                "us_per_launch": round(t / (n * launches_per_layer) * 1e6, 3),
+                "layers_timed": n,
+            }
+            del g
+        return table
+
+    per_width = width_table(grouped=True)          # 1 launch per layer and width
+    per_width_dropin = width_table(grouped=False)  # 7 launches per layer and width
+
+    # drop-in, all three widths (the reference's launch structure: 21 launches per step)
+    n_d = graph_steps(step_bytes)
+    run.cursor = 0
+    gd = run.capture(n_d, WIDTHS, grouped=False)
+    gd.replay()
+    torch.cuda.synchronize()
+    t_d, t_d_med = run.time_stats(gd)
+    drop_in = {
+        "gbps": round(step_bytes * n_d / t_d / 1e9, 1),
+        "pct_hbm_peak": round(step_bytes * n_d / t_d / 1e9 / HBM_PEAK_GBPS * 100, 2),
+        "ms_per_step": round(t_d / n_d * 1e3, 5), "launches_per_step": len(WIDTHS) * len(PROJECTIONS),
+        "per_width": {str(m): per_width_dropin[m] for m in WIDTHS},
+    }
+    del gd
 
     # the same layer bytes in the four merged matrices the decode step launches
     # (q|k|v and gate|up concatenated along N, as the reference's prepare_merged_weights,
-    # model.py:931-956,1042-1051): 4 launches per layer instead of 7
+    # model.py:931-956,1042-1051): 4 drop-in launches per layer instead of 7
     merged_shapes = ((4096, 2048, (0, 1, 2)), (2048, 2048, (3,)), (12288, 2048, (4, 5)),
                      (2048, 6144, (6,)))
     mpool = [[(torch.cat([layer[i][0] for i in idx]).contiguous(),
@@ -299,11 +348,12 @@ def main() -> int:
     mouts = {(m, j): torch.empty(m, n, dtype=torch.bfloat16, device=dev)
              for m in WIDTHS for j, (n, _, _) in enumerate(merged_shapes)}
     merged = {}
+    n_m = graph_steps(LAYER_BYTES)
     for m in WIDTHS:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             spc = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            for st in range(args.steps):
+            for st in range(n_m):
                 layer = mpool[st % len(mpool)]
                 for j, (n, k, _) in enumerate(merged_shapes):
                     q, s_ = acts[(m, k)]
@@ -311,42 +361,28 @@ def main() -> int:
                            s_.data_ptr(), layer[j][1].data_ptr(), m, n, k, spc)
         g.replay()
         torch.cuda.synchronize()
-        t = min(run.time_graph(g) for _ in range(3))
+        t, _ = run.time_stats(g)
         merged[str(m)] = {
-            "gbps": round(LAYER_BYTES * args.steps / t / 1e9, 1),
-            "pct_hbm_peak": round(LAYER_BYTES * args.steps / t / 1e9 / HBM_PEAK_GBPS * 100, 2),
-            "us_per_layer": round(t / args.steps * 1e6, 3),
-            "us_per_launch": round(t / (args.steps * len(merged_shapes)) * 1e6, 3),
+            "gbps": round(LAYER_BYTES * n_m / t / 1e9, 1),
+            "pct_hbm_peak": round(LAYER_BYTES * n_m / t / 1e9 / HBM_PEAK_GBPS * 100, 2),
+            "us_per_layer": round(t / n_m * 1e6, 3),
+            "us_per_launch": round(t / (n_m * len(merged_shapes)) * 1e6, 3),
         }
         del g
     del mpool
 
-    # secondary figure: the same 21 launches per step on four forked streams of one graph
-    # (two launches may write the same output buffer at once: the values are not used)
-    run.cursor = 0
-    gc_ = run.capture_concurrent(args.steps, WIDTHS, 4)
-    gc_.replay()
-    torch.cuda.synchronize()
-    t_conc = min(run.time_graph(gc_) for _ in range(3))
-    concurrent = {
-        "streams": 4, "gbps": round(step_bytes * args.steps / t_conc / 1e9, 1),
-        "pct_hbm_peak": round(step_bytes * args.steps / t_conc / 1e9 / HBM_PEAK_GBPS * 100, 2),
-        "us_per_launch": round(t_conc / (args.steps * len(WIDTHS) * len(PROJECTIONS)) * 1e6, 3),
-        "note": "independent projections overlapped; `value` is the serial figure",
-    }
-    del gc_
-
-    # roofline of the dominant kernel: the width whose launches take the most time
+    # roofline of the dominant kernel: the grouped matrix-core kernel at the width whose
+    # launches take the most time; one launch streams one layer (13,369,344 algorithmic bytes)
     dom = max(WIDTHS, key=lambda m: per_width[m]["us_per_launch"])
-    bytes_per_launch = LAYER_BYTES / len(PROJECTIONS)
+    bytes_per_launch = LAYER_BYTES
     achieved = bytes_per_launch / (per_width[dom]["us_per_launch"] * 1e-6) / 1e9
+    traffic = measured_traffic(dom)
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": round(MEASURED_TRAFFIC_BYTES[dom]),
-        "kernel": (f"gemv_mfma_direct_kernel<BITS=2> (width {dom})" if dom >= 3
-                   else f"gemv_dot4_kernel<BITS=2, MT={dom}> (width {dom})"),
-        "bytes_per_launch": round(bytes_per_launch),
+        "traffic": None if traffic is None else round(traffic),
+        "kernel": f"gemv_mx_kernel<BITS=2, R=1> (grouped, 7 descriptors, width {dom})",
+        "bytes_per_launch": bytes_per_launch,
         "us_per_launch": per_width[dom]["us_per_launch"],
     }
 
@@ -384,7 +420,7 @@ def main() -> int:
     # 1.7B-shaped model (configs[2]), AR and D8 hybrid, by the reference's timing contract.
     decode = decode_bf16 = decode_4b = None
     if not args.no_decode:
-        del run, pool, graph
+        del run, pool
         torch.cuda.empty_cache()
         from bitmtp_amd.decode_bench import run_decode_bench
         decode = run_decode_bench("1.7b", prompt_len=256, new_tokens=512, repeats=1)
@@ -406,14 +442,18 @@ def main() -> int:
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {
             "workload": "configs[1]: 7 T2-g128 projections of one Qwen3-1.7B-shaped layer at "
-                        "widths 1,4,8 (21 launches/step), HBM-cold over a pool of distinct layers",
+                        "widths 1,4,8, grouped: one t2g128_gemv_grouped launch per width "
+                        "(3 launches/step), HBM-cold over a pool of distinct layers",
             "pool_layers": args.layers, "pool_bytes": args.layers * LAYER_BYTES,
-            "bytes_per_step": step_bytes, "launches_per_step": len(WIDTHS) * len(PROJECTIONS),
+            "bytes_per_step": step_bytes, "launches_per_step": len(WIDTHS),
+            "steps_in_timed_graph": n_g, "seconds_for_steps": round(elapsed, 6),
             "pct_hbm_peak": round(gbps / HBM_PEAK_GBPS * 100, 2),
+            "median_pct_hbm_peak": round(headline_median_gbps / HBM_PEAK_GBPS * 100, 2),
             "per_width": {str(m): per_width[m] for m in WIDTHS},
-            "timing": "one HIP graph of all steps, HIP events on the launch stream, best of 3 replays",
+            "timing": "one HIP graph per figure holding >= 512 MB of distinct weights, HIP events "
+                      "on the launch stream, best and median of 5 replays",
+            "drop_in": drop_in,
             "merged_decode_shapes_4_launches_per_layer": merged,
-            "concurrent_streams": concurrent,
             "lm_head_151936x2048": head,
             "decode_1p7b_d8": decode,
             "decode_1p7b_d8_bf16_lm_head": decode_bf16,
