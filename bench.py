@@ -246,9 +246,16 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true",
                     help="skip the end-to-end decode tokens/s section")
     ap.add_argument("--no-head", action="store_true", help="skip the lm_head-sized extra measurement")
+    ap.add_argument("--widths", default=None,
+                    help="comma list restricting the widths measured (profiling runs); default 1,4,8")
+    ap.add_argument("--no-drop-in", action="store_true",
+                    help="skip the one-launch-per-projection and merged-matrix figures (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device copy (for scaling rocprofv3 PMC byte counters)")
     args = ap.parse_args()
+    global WIDTHS
+    if args.widths:
+        WIDTHS = tuple(int(w) for w in args.widths.split(","))
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (--gpus must be 1)",
               file=sys.stderr)
@@ -320,22 +327,26 @@ def main() -> int:
         return table
 
     per_width = width_table(grouped=True)          # 1 launch per layer and width
-    per_width_dropin = width_table(grouped=False)  # 7 launches per layer and width
+    skip_drop_in = args.no_drop_in
+    per_width_dropin = {} if skip_drop_in else width_table(grouped=False)  # 7 launches per layer
 
     # drop-in, all three widths (the reference's launch structure: 21 launches per step)
-    n_d = graph_steps(step_bytes)
-    run.cursor = 0
-    gd = run.capture(n_d, WIDTHS, grouped=False)
-    gd.replay()
-    torch.cuda.synchronize()
-    t_d, t_d_med = run.time_stats(gd)
-    drop_in = {
-        "gbps": round(step_bytes * n_d / t_d / 1e9, 1),
-        "pct_hbm_peak": round(step_bytes * n_d / t_d / 1e9 / HBM_PEAK_GBPS * 100, 2),
-        "ms_per_step": round(t_d / n_d * 1e3, 5), "launches_per_step": len(WIDTHS) * len(PROJECTIONS),
-        "per_width": {str(m): per_width_dropin[m] for m in WIDTHS},
-    }
-    del gd
+    drop_in, merged = None, {}
+    n_d = 0 if skip_drop_in else graph_steps(step_bytes)
+    if not skip_drop_in:
+        run.cursor = 0
+        gd = run.capture(n_d, WIDTHS, grouped=False)
+        gd.replay()
+        torch.cuda.synchronize()
+        t_d, t_d_med = run.time_stats(gd)
+        drop_in = {
+            "gbps": round(step_bytes * n_d / t_d / 1e9, 1),
+            "pct_hbm_peak": round(step_bytes * n_d / t_d / 1e9 / HBM_PEAK_GBPS * 100, 2),
+            "ms_per_step": round(t_d / n_d * 1e3, 5),
+            "launches_per_step": len(WIDTHS) * len(PROJECTIONS),
+            "per_width": {str(m): per_width_dropin[m] for m in WIDTHS},
+        }
+        del gd
 
     # the same layer bytes in the four merged matrices the decode step launches
     # (q|k|v and gate|up concatenated along N, as the reference's prepare_merged_weights,
@@ -347,9 +358,8 @@ def main() -> int:
               for _, _, idx in merged_shapes] for layer in pool]
     mouts = {(m, j): torch.empty(m, n, dtype=torch.bfloat16, device=dev)
              for m in WIDTHS for j, (n, _, _) in enumerate(merged_shapes)}
-    merged = {}
     n_m = graph_steps(LAYER_BYTES)
-    for m in WIDTHS:
+    for m in (() if skip_drop_in else WIDTHS):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             spc = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
