@@ -17,6 +17,7 @@
 #include "gemv_fp4.hip.h"
 #include "gemv_mfma.hip.h"
 #include "gemv_mx.hip.h"
+#include "gemv_mxs.hip.h"
 #include "packed_gemv.hip.h"
 
 namespace bonsai {
@@ -39,6 +40,8 @@ int init_all_kernels() {
         if (rc3 != 0) return rc3;
         const int rc4 = mx_init_device<BITS>(st.lds_limit[dev]);
         if (rc4 != 0) return rc4;
+        const int rc5 = mxs_init_device<BITS>(st.lds_limit[dev]);
+        if (rc5 != 0) return rc5;
         int cus = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
             cus <= 0)
@@ -207,6 +210,12 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     const MfmaTuning &mtu = mfma_tuning<BITS>();
     const int min_width = mtu.min_width > 0 ? mtu.min_width
                                             : (N >= kLongMatrixRows ? 2 : kDefaultMfmaMinWidth);
+    if (mtu.engine == 5 || mtu.engine == 0) {
+        // very long matrices: the streaming kernel, at every width up to 16
+        const GemvProblem q{A, B, out, s, ws, M, N, K};
+        if (mxs_problem_ok<BITS>(q, out_kind, lds_limit, st.n_cus[dev], mtu.engine == 5))
+            return launch_mxs<BITS>(q, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
+    }
     if (mtu.engine == 4 && M >= min_width) {
         // the grouped kernel with a single descriptor
         const GemvProblem q{A, B, out, s, ws, M, N, K};

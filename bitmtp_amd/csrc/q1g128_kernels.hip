@@ -113,6 +113,12 @@ void q1g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width) {
     t.min_width = min_width;
 }
 
+void q1g128_set_stream_tuning(int min_bytes, int wgs_per_cu) {
+    MxsTuning &t = mxs_tuning<1>();
+    t.min_bytes = min_bytes;
+    t.wgs_per_cu = wgs_per_cu;
+}
+
 int q1g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
                    int M, int N, int K, int out_kind, int scale_kind, void *stream) {
     return launch_gemv<1>(A, B, out, s, ws, M, N, K, out_kind, scale_kind,

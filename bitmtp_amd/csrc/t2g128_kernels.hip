@@ -44,6 +44,12 @@ void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width) {
     t.min_width = min_width;
 }
 
+void t2g128_set_stream_tuning(int min_bytes, int wgs_per_cu) {
+    MxsTuning &t = mxs_tuning<2>();
+    t.min_bytes = min_bytes;
+    t.wgs_per_cu = wgs_per_cu;
+}
+
 int t2g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s, const void *ws,
                    int M, int N, int K, int out_kind, int scale_kind, void *stream) {
     return launch_gemv<2>(A, B, out, s, ws, M, N, K, out_kind, scale_kind,

@@ -89,6 +89,8 @@ def load_t2_kernel() -> None:
     lib.t2g128_gemv_grouped.restype = ctypes.c_int
     lib.t2g128_set_grouped_tuning.argtypes = [ctypes.c_int] * 3
     lib.t2g128_set_grouped_tuning.restype = None
+    lib.t2g128_set_stream_tuning.argtypes = [ctypes.c_int] * 2
+    lib.t2g128_set_stream_tuning.restype = None
     _t2_lib = lib
 
 
@@ -115,6 +117,8 @@ def load_q1_kernel() -> None:
     lib.q1g128_gemv_grouped.restype = ctypes.c_int
     lib.q1g128_set_grouped_tuning.argtypes = [ctypes.c_int] * 3
     lib.q1g128_set_grouped_tuning.restype = None
+    lib.q1g128_set_stream_tuning.argtypes = [ctypes.c_int] * 2
+    lib.q1g128_set_stream_tuning.restype = None
     _q1_lib = lib
 
 
@@ -267,10 +271,12 @@ def packed_int8_linear(a_int8, b_packed, s, ws):
 
 
 def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[torch.Tensor],
-                   ws: Optional[torch.Tensor], *, bits: int, out_kind: int = OUT_BF16) -> torch.Tensor:
+                   ws: Optional[torch.Tensor], *, bits: int, out_kind: int = OUT_BF16,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same kernels with a selectable result: bf16 ``[M,N]``, the fp32 value
     before the bf16 rounding, or the exact int32 group sums ``[M,N,K/128]``.
-    ``ws`` may be bf16 or fp16.  Rank-2 activations only."""
+    ``ws`` may be bf16 or fp16.  Rank-2 activations only.  ``out`` supplies a preallocated
+    result (so that a captured graph allocates nothing)."""
     if bits not in (1, 2):
         raise ValueError("bits must be 1 (Q1) or 2 (T2)")
     kind = "t2g128" if bits == 2 else "q1"
@@ -293,13 +299,18 @@ def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[tor
     m, n, k = a_int8.shape[0], b_packed.shape[0], b_packed.shape[1] * (8 // bits)
     dev = a_int8.device
     if out_kind == OUT_BF16:
-        out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+        shape, dtype = (m, n), torch.bfloat16
     elif out_kind == OUT_F32:
-        out = torch.empty(m, n, dtype=torch.float32, device=dev)
+        shape, dtype = (m, n), torch.float32
     elif out_kind == OUT_G32:
-        out = torch.empty(m, n, k // 128, dtype=torch.int32, device=dev)
+        shape, dtype = (m, n, k // 128), torch.int32
     else:
         raise ValueError("bad out_kind")
+    if out is None:
+        out = torch.empty(*shape, dtype=dtype, device=dev)
+    elif (tuple(out.shape) != shape or out.dtype != dtype or out.device != dev
+          or not out.is_contiguous()):
+        raise RuntimeError(f"{kind}: out must be a contiguous {dtype} tensor of shape {shape} on {dev}")
     scale_kind = SCALE_F16 if (ws is not None and ws.dtype == torch.float16) else SCALE_BF16
     fn = t2_lib().t2g128_gemv_ex if bits == 2 else q1_lib().q1g128_gemv_ex
     with torch.cuda.device(dev):

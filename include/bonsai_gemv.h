@@ -118,27 +118,6 @@ int q1g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, 
 int t2g128_init(void);
 int q1g128_init(void);
 
-/* Launch-geometry override for tuning experiments: lanes per weight row
- * (4..64, power of two), waves per workgroup (1..16) and row passes per wave
- * (>= 1).  Zero restores the built-in heuristic for that field.  Process-wide,
- * not thread-safe; no reference counterpart. */
-void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
-void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
-
-/* The same for the matrix-core kernels that serve widths >= min_width: smallest
- * width they take (a value above any M disables them), 16-row tiles per wave (1,
- * 2 or 4), waves of a workgroup splitting K (1, 2 or 4), row blocks a workgroup
- * walks through (used when K is not split) and the engine (2 = FP4 x FP8 MFMA,
- * otherwise int8 MFMA).  Zero = built-in choice. */
-void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
-void q1g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
-
-/* Development hook of the grouped kernel: 16-row tiles per wave (1 or 2), cap on the
- * workgroups of one launch, smallest width sent to it.  Zero = built-in choice.  Process-wide,
- * not thread-safe. */
-void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
-void q1g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
-
 /* ---- activation quantisation (libbonsai_actq.so) ------------------------- */
 /* Per-token symmetric INT8 quantisation, the native form of `quant_input`
  * (src/bonsai_sft/gpu/model.py:632-636, identical copy at :571-575):
@@ -179,6 +158,34 @@ int bonsai_add_rmsnorm_bf16(const void *x, const void *residual, const void *w, 
  * columns [0,F) and up in [F,2F); inner = bf16(bf16(silu(gate)) * up); q int8
  * [M,F], s fp32 [M]. */
 int bonsai_silu_mul_quant_int8(const void *gate_up, int8_t *q, float *s, int M, int F, void *stream);
+
+/* ---- development hooks --------------------------------------------------------- */
+/* Overrides of the built-in kernel choice and launch geometry, for measurements and for the
+ * tests that force every kernel onto small shapes.  Not part of the drop-in surface: no
+ * reference counterpart, process-wide, not thread-safe, and a value of zero always restores
+ * the built-in choice for that field.  Results never depend on them (every kernel computes the
+ * arithmetic stated at the top of this file); only speed does.
+ *
+ * set_tuning: the dot4 kernel -- lanes per weight row (4..64, power of two), waves per
+ *   workgroup (1..16), row passes per wave (>= 1).
+ * set_mfma_tuning: the single-GEMV matrix-core kernels -- smallest width they take (a value
+ *   above any M disables them); 16-row tiles per wave (1, 2 or 4); waves of a workgroup that
+ *   split K (1, 2, 4, 8, or 3..12 for the one-tile-per-wave form); row blocks a workgroup walks
+ *   when K is not split; engine: 1 = int8 MFMA with activations staged in LDS, 3 = int8 MFMA
+ *   with activations loaded as operands, 4 = the grouped kernel with one descriptor,
+ *   5 = the streaming kernel on any shape it can run (otherwise only on very long matrices).
+ * set_grouped_tuning: the grouped kernel -- 16-row tiles per wave (1 or 2), cap on the
+ *   workgroups of one launch, smallest width sent to it.
+ * set_stream_tuning: the streaming kernel for very long matrices -- smallest packed size in
+ *   bytes that is sent to it (negative: never), persistent workgroups per CU. */
+void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
+void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
+void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
+void q1g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);
+void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
+void q1g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
+void t2g128_set_stream_tuning(int min_bytes, int wgs_per_cu);
+void q1g128_set_stream_tuning(int min_bytes, int wgs_per_cu);
 
 #ifdef __cplusplus
 }

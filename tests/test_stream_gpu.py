@@ -1,0 +1,102 @@
+"""GPU parity of the streaming matrix-core kernel (the one very long matrices such as the packed
+lm_head take) against the CPU oracle, through the C ABI.  The kernel is forced on shapes the
+oracle finishes in seconds (engine 5 of the tuning call) and checked at the full head shape through
+the ordinary entry point: fp32 value within rtol 1e-3 / atol 1e-3, bf16 output the oracle's or the
+neighbouring representable value and equal to the RNE rounding of the fp32 value.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import bf16_bits, bf16_ordinal, to_dev
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-3
+ATOL = 1e-3
+
+
+def check_one(O, p, bits, label, scale_kind=0):
+    import bitmtp_amd as ops
+    A, B, s, ws = to_dev(p)
+    print(f"[case] stream {label} bits={bits} M={p['A'].shape[0]} N={p['B'].shape[0]} K={p['A'].shape[1]}",
+          flush=True)
+    y32 = ops.packed_gemv_ex(A, B, s, ws, bits=bits, out_kind=ops.OUT_F32)
+    y16 = ops.packed_gemv_ex(A, B, s, ws, bits=bits, out_kind=ops.OUT_BF16)
+    torch.cuda.synchronize()
+    y32_ref, y16_ref = O.c_gemv(p["A"], p["B"], p["s"], p["ws"], bits)
+    got = y32.cpu().numpy()
+    err = np.abs(got - y32_ref)
+    assert np.all(err <= ATOL + RTOL * np.abs(y32_ref)), f"{label}: fp32 max err {err.max()}"
+    d = np.abs(bf16_ordinal(bf16_bits(y16)) - bf16_ordinal(y16_ref))
+    assert d.max() <= 1, f"{label}: bf16 output more than one representable value away"
+    assert np.array_equal(bf16_bits(y16), O.f32_to_bf16_bits(got)), f"{label}: bf16 != rne(fp32)"
+
+
+@pytest.fixture
+def forced_stream():
+    from bitmtp_amd import ops as O2
+    t2, q1 = O2.t2_lib(), O2.q1_lib()
+    t2.t2g128_set_mfma_tuning(0, 0, 0, 0, 5)
+    q1.q1g128_set_mfma_tuning(0, 0, 0, 0, 5)
+    yield (t2, q1)
+    t2.t2g128_set_mfma_tuning(0, 0, 0, 0, 0)
+    q1.q1g128_set_mfma_tuning(0, 0, 0, 0, 0)
+    t2.t2g128_set_stream_tuning(0, 0)
+    q1.q1g128_set_stream_tuning(0, 0)
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+@pytest.mark.parametrize("M,N,K", [
+    (1, 4096, 2048), (8, 4099, 2048), (9, 1000, 2048), (16, 257, 2048), (5, 33, 2560), (3, 8200, 2560),
+    (2, 15, 4096), (16, 700, 3072), (7, 1, 2048), (12, 20000, 2048),
+])
+def test_forced_stream_kernel(oracle, forced_stream, bits, M, N, K):
+    """Ragged row counts, K / 512 that is no multiple of the ring depth (the stream then ends
+    inside a trip), fewer row tiles than waves, blocks of up to 16 tokens."""
+    check_one(oracle, oracle.synth_problem(1000 + M + N, M, N, K, bits), bits, "forced")
+
+
+@pytest.mark.parametrize("wgs_per_cu", [1, 2, 3])
+def test_forced_stream_kernel_other_residency(oracle, forced_stream, wgs_per_cu):
+    forced_stream[0].t2g128_set_stream_tuning(0, wgs_per_cu)
+    check_one(oracle, oracle.synth_problem(1100 + wgs_per_cu, 8, 40000, 2048, 2), 2, f"wgs/cu {wgs_per_cu}")
+
+
+def test_forced_stream_kernel_extreme_bytes(oracle, forced_stream):
+    rng = np.random.default_rng(11)
+    p = oracle.synth_problem(1200, 6, 600, 2048, 2)
+    p["A"] = rng.integers(-128, 128, size=p["A"].shape, dtype=np.int8)
+    p["A"][0, :] = -128
+    p["B"] = rng.integers(0, 256, size=p["B"].shape, dtype=np.uint8)
+    p["B"][0, :] = 0x00
+    p["B"][1, :] = 0xFF
+    check_one(oracle, p, 2, "extreme")
+
+
+@pytest.mark.parametrize("M", [1, 4, 9, 16])
+def test_head_shape_default_dispatch(oracle, M):
+    """The 151936 x 2048 packed lm_head through the ordinary entry point."""
+    check_one(oracle, oracle.synth_problem(1300 + M, M, 151936, 2048, 2), 2, "head")
+
+
+def test_head_shape_4b(oracle):
+    check_one(oracle, oracle.synth_problem(1400, 8, 151936, 2560, 2), 2, "head 4B")
+
+
+def test_stream_kernel_graph_replay(oracle):
+    import bitmtp_amd as ops
+    ops.init_kernels()
+    A, B, s, ws = to_dev(oracle.synth_problem(1500, 8, 151936, 2048, 2))
+    eager = ops.packed_gemv_ex(A, B, s, ws, bits=2).clone()
+    out = torch.empty_like(eager)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        ops.packed_gemv_ex(A, B, s, ws, bits=2, out=out)
+    for rep in range(3):
+        out.zero_()
+        _ = ops.packed_gemv_ex(A, B, s, ws, bits=2)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs"
