@@ -26,6 +26,126 @@ constexpr int kDefaultMfmaMinWidth = 3;       // layer-sized matrices (dot4 wins
 constexpr int kDirectMaxRows = 16384;         // up to here the staging-free matrix-core kernel
 constexpr int kLongMatrixRows = 32768;        // from here on the matrix cores pay off at M >= 2
 
+// ---- grouped dot4 launch (narrow blocks) -------------------------------------------------
+constexpr int kDot4GroupMaxWidth = 2;  // widest block the grouped dot4 kernel takes
+
+using Dot4GroupFn = void (*)(int, int, int, int, int, int, int, int, int, int, int, int, int, int,
+                             const Dot4GroupTable);
+
+template <int BITS>
+struct Dot4GroupKernels {
+    Dot4GroupFn fn[kDot4GroupMaxWidth][kBatchKinds][2];  // [MT - 1][U index][scale kind]
+};
+
+template <int BITS>
+const Dot4GroupKernels<BITS> &dot4_group_kernels() {
+    static const Dot4GroupKernels<BITS> t = [] {
+        Dot4GroupKernels<BITS> x{};
+        x.fn[0][0][0] = gemv_dot4_grouped_kernel<BITS, 1, 1, false>;
+        x.fn[0][0][1] = gemv_dot4_grouped_kernel<BITS, 1, 1, true>;
+        x.fn[0][1][0] = gemv_dot4_grouped_kernel<BITS, 1, 2, false>;
+        x.fn[0][1][1] = gemv_dot4_grouped_kernel<BITS, 1, 2, true>;
+        x.fn[0][2][0] = gemv_dot4_grouped_kernel<BITS, 1, 4, false>;
+        x.fn[0][2][1] = gemv_dot4_grouped_kernel<BITS, 1, 4, true>;
+        x.fn[1][0][0] = gemv_dot4_grouped_kernel<BITS, 2, 1, false>;
+        x.fn[1][0][1] = gemv_dot4_grouped_kernel<BITS, 2, 1, true>;
+        x.fn[1][1][0] = gemv_dot4_grouped_kernel<BITS, 2, 2, false>;
+        x.fn[1][1][1] = gemv_dot4_grouped_kernel<BITS, 2, 2, true>;
+        x.fn[1][2][0] = gemv_dot4_grouped_kernel<BITS, 2, 4, false>;
+        x.fn[1][2][1] = gemv_dot4_grouped_kernel<BITS, 2, 4, true>;
+        return x;
+    }();
+    return t;
+}
+
+template <int BITS>
+int dot4_group_init_device(int max_lds) {
+    const Dot4GroupKernels<BITS> &t = dot4_group_kernels<BITS>();
+    for (int mt = 0; mt < kDot4GroupMaxWidth; ++mt)
+        for (int u = 0; u < kBatchKinds; ++u)
+            for (int sk = 0; sk < 2; ++sk)
+                if (hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[mt][u][sk]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        max_lds) != hipSuccess)
+                    return 2;
+    return 0;
+}
+
+// Launches up to kDot4GroupMax problems of at most kDot4GroupMaxWidth tokens each with the
+// grouped dot4 kernel.  Lanes per row and passes are each problem's own (pick_geometry); the
+// token tile, the loads per batch and the workgroup size are common to the launch (the widest
+// block, the shortest batch and the smaller workgroup any problem asks for).  Returns 0, -1
+// when a problem does not fit (the caller falls back), 2 on a launch error.
+template <int BITS>
+int launch_dot4_grouped(const GemvProblem *probs, int count, int out_kind, int scale_kind,
+                        int lds_limit, hipStream_t stream) {
+    if (count < 1 || count > kDot4GroupMax || out_kind == OUT_G32) return -1;
+    int mt = 1;
+    for (int i = 0; i < count; ++i) mt = probs[i].M > mt ? probs[i].M : mt;
+    if (mt > kDot4GroupMaxWidth) return -1;
+    // longest rows first: their workgroups run longest and should start first
+    int order[kDot4GroupMax];
+    for (int i = 0; i < count; ++i) order[i] = i;
+    for (int i = 1; i < count; ++i)
+        for (int j = i; j > 0 && probs[order[j]].K > probs[order[j - 1]].K; --j) {
+            const int t = order[j];
+            order[j] = order[j - 1];
+            order[j - 1] = t;
+        }
+    Geometry geo[kDot4GroupMax];
+    int waves = 8, batch_index = kBatchKinds - 1;
+    size_t lds = 0;
+    // A launch of several matrices has waves enough without spreading every row over many
+    // lanes: at most sixteen lanes per row with at least two loads each, four waves per
+    // workgroup (sweep over the seven projections of the 1.7B-shaped layer, one token:
+    // 5.65 us against 6.4 us with each matrix's own single-launch geometry).
+    Tuning tu = lib_state<BITS>().tuning;
+    const bool own_rule = tu.lanes_per_row == 0 && tu.waves_per_wg == 0 && count > 1;
+    for (int i = 0; i < count; ++i) {
+        const GemvProblem &q = probs[order[i]];
+        Tuning t = tu;
+        if (own_rule) {
+            const int C = q.K / Fmt<BITS>::kChunkWeights;
+            int lpr = BITS == 1 ? 4 : 8;
+            while (lpr < 16 && 2 * lpr * 2 <= C) lpr *= 2;
+            t.lanes_per_row = lpr;
+            t.waves_per_wg = 4;
+        }
+        geo[i] = pick_geometry<BITS>(mt, q.N, q.K, lds_limit, t);
+        if (geo[i].mt != mt) return -1;  // the token tile does not fit the LDS
+        waves = geo[i].waves < waves ? geo[i].waves : waves;
+        batch_index = geo[i].batch_index < batch_index ? geo[i].batch_index : batch_index;
+        lds = geo[i].lds > lds ? geo[i].lds : lds;
+    }
+    Dot4GroupTable tbl{};
+    int ends[kDot4GroupMax];
+    int wg = 0;
+    for (int i = 0; i < count; ++i) {
+        const GemvProblem &q = probs[order[i]];
+        Dot4GroupDesc &d = tbl.d[i];
+        d.A = q.A;
+        d.B = q.B;
+        d.out = q.out;
+        d.s = q.s;
+        d.ws = reinterpret_cast<const uint16_t *>(q.ws);
+        d.M = q.M;
+        d.N = q.N;
+        d.K = q.K;
+        d.wg_begin = wg;
+        d.lpr_log2_passes = geo[i].lpr_log2 | (geo[i].passes << 8);
+        d.div_magic = (uint32_t)(0x100000000ull / (uint64_t)(4 * (q.K / Fmt<BITS>::kChunkWeights))) + 1u;
+        const long rows_per_wg = (long)(64 >> geo[i].lpr_log2) * waves * geo[i].passes;
+        wg += (int)(((long)q.N + rows_per_wg - 1) / rows_per_wg);
+        ends[i] = wg;
+    }
+    for (int i = count; i < kDot4GroupMax; ++i) ends[i] = 0x7fffffff;
+    const Dot4GroupFn fn = dot4_group_kernels<BITS>().fn[mt - 1][batch_index][scale_kind];
+    hipLaunchKernelGGL(fn, dim3(wg, 1, 1), dim3(waves * 64, 1, 1), lds, stream, ends[0], ends[1],
+                       ends[2], ends[3], ends[4], ends[5], ends[6], ends[7], ends[8], ends[9],
+                       ends[10], ends[11], out_kind == OUT_F32 ? 1 : 0, waves * 64, tbl);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
 template <int BITS>
 int init_all_kernels() {
     const int rc = init_device<BITS>();
@@ -42,6 +162,8 @@ int init_all_kernels() {
         if (rc4 != 0) return rc4;
         const int rc5 = mxs_init_device<BITS>(st.lds_limit[dev]);
         if (rc5 != 0) return rc5;
+        const int rc6 = dot4_group_init_device<BITS>(st.lds_limit[dev]);
+        if (rc6 != 0) return rc6;
         int cus = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
             cus <= 0)
@@ -277,9 +399,34 @@ int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_
         nb = 0;
         return rc;
     };
+    // Blocks of one or two tokens: the grouped dot4 kernel, twelve problems per launch
+    // (a forced smallest width of the matrix-core kernel, tu.min_width > 0, keeps them there)
+    GemvProblem nbatch[kDot4GroupMax];
+    int nnb = 0;
+    const bool narrow_on = out_kind != OUT_G32 && tu.min_width <= 0;
+    auto flush_n = [&]() -> int {
+        if (nnb == 0) return 0;
+        int rc = launch_dot4_grouped<BITS>(nbatch, nnb, out_kind, scale_kind, lds_limit, stream);
+        if (rc == -1) {  // did not fit: one by one
+            rc = 0;
+            for (int i = 0; i < nnb && rc == 0; ++i)
+                rc = launch_gemv<BITS>(nbatch[i].A, nbatch[i].B, nbatch[i].out, nbatch[i].s, nbatch[i].ws,
+                                       nbatch[i].M, nbatch[i].N, nbatch[i].K, out_kind, scale_kind, stream);
+        }
+        nnb = 0;
+        return rc;
+    };
     const size_t out_elt = out_kind == OUT_BF16 ? 2 : 4;
     for (int i = 0; i < count; ++i) {
         const GemvProblem &q = probs[i];
+        if (narrow_on && q.M <= kDot4GroupMaxWidth) {
+            nbatch[nnb++] = q;
+            if (nnb == kDot4GroupMax) {
+                const int rc = flush_n();
+                if (rc != 0) return rc;
+            }
+            continue;
+        }
         // token tiles of at most 16 (the staged activations are chunked along K: they always fit)
         const int cap = q.M < kMfmaTokens ? q.M : kMfmaTokens;
         if (q.M < min_width || !mx_problem_ok(q, out_kind == OUT_G32)) {
@@ -304,6 +451,8 @@ int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_
             }
         }
     }
+    const int rcn = flush_n();
+    if (rcn != 0) return rcn;
     const int rc = flush();
     return rc < 0 ? 2 : rc;
 }

@@ -99,15 +99,11 @@ struct WeightBatch {
 // BITS: 2 = T2, 1 = Q1.  MT: tokens in the tile.  U: 16-byte weight loads a lane
 // issues back to back (one batch).  G32: write the int32 group sums instead of
 // the scaled result.  SF16: group scales are fp16 instead of bf16.
+// The kernel proper: workgroup `bx` of the GEMV `a`, token tile `by`, `pthreads` threads.
 template <int BITS, int MT, int U, bool G32, bool SF16>
-__global__ void __launch_bounds__(kMaxThreads)
-gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *ps,
-                 const uint16_t *pws, int pM, int pN, int pK, int plpr_log2, int ppasses,
-                 int pout_f32, uint32_t pdiv_magic, int pthreads) {
-    // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
-    const GemvArgs a{pA, pB, pout, ps, pws, pM, pN, pK, plpr_log2, ppasses, pout_f32, pdiv_magic};
+__device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by, int pthreads,
+                                               unsigned char *smem) {
     using F = Fmt<BITS>;
-    extern __shared__ __align__(16) unsigned char smem[];
 
     const int K = a.K, N = a.N, M = a.M;
     const int C = K / F::kChunkWeights;  // 16-byte chunks per weight row
@@ -128,8 +124,8 @@ gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *p
     const int rpw = 64 >> lpr_log2;  // rows per wave and pass
     const int IT = (C + lpr - 1) >> lpr_log2;
     const int nb = (IT + U - 1) / U;
-    const int m0 = blockIdx.y * MT;
-    const int row0 = ((int)blockIdx.x * a.passes * nwaves + wave) * rpw + r;
+    const int m0 = by * MT;
+    const int row0 = (bx * a.passes * nwaves + wave) * rpw + r;
     const int row_step = nwaves * rpw;  // rows between two passes of a wave
 
     // All loads of a batch are unconditional (indices clamped into the row) and
@@ -283,6 +279,61 @@ gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *p
     } else {
         compute_batch(cur, pa, ba);
     }
+}
+
+template <int BITS, int MT, int U, bool G32, bool SF16>
+__global__ void __launch_bounds__(kMaxThreads)
+gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *ps,
+                 const uint16_t *pws, int pM, int pN, int pK, int plpr_log2, int ppasses,
+                 int pout_f32, uint32_t pdiv_magic, int pthreads) {
+    // scalar parameters (instead of one struct) so that they can be preloaded into SGPRs
+    const GemvArgs a{pA, pB, pout, ps, pws, pM, pN, pK, plpr_log2, ppasses, pout_f32, pdiv_magic};
+    extern __shared__ __align__(16) unsigned char smem[];
+    gemv_dot4_body<BITS, MT, U, G32, SF16>(a, (int)blockIdx.x, (int)blockIdx.y, pthreads, smem);
+}
+
+// ---- several GEMVs in one launch -------------------------------------------------------
+// The same kernel over a table of up to twelve GEMVs: a workgroup finds its GEMV by comparing
+// its number with the range ends, which arrive in SGPRs with the wave (preloaded kernel
+// arguments), reads that GEMV's 64-byte descriptor with one scalar load and runs the body.
+// For narrow blocks (one or two tokens) this is the fastest grouped form: no cross-wave
+// reduction, a row's lanes add up on the DPP network, and a wave's critical path after its
+// weights arrive is one batch of dot products.  Launches of one kernel per projection are what
+// it replaces (src/bonsai_sft/gpu/model.py:977-1062).
+constexpr int kDot4GroupMax = 12;
+
+struct Dot4GroupDesc {
+    const int8_t *A;
+    const uint8_t *B;
+    void *out;
+    const float *s;
+    const uint16_t *ws;
+    int M, N, K;
+    int wg_begin;         // first workgroup of this GEMV
+    int lpr_log2_passes;  // lpr_log2 | passes << 8
+    uint32_t div_magic;
+};
+static_assert(sizeof(Dot4GroupDesc) == 64, "one descriptor is one 64-byte scalar load");
+
+struct Dot4GroupTable {
+    Dot4GroupDesc d[kDot4GroupMax];
+};
+
+template <int BITS, int MT, int U, bool SF16>
+__global__ void __launch_bounds__(kMaxThreads)
+gemv_dot4_grouped_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, int e8,
+                         int e9, int e10, int e11, int pout_f32, int pthreads,
+                         const Dot4GroupTable tbl) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int wg = (int)blockIdx.x;
+    // (wg >= e) as the sign bit of e - 1 - wg: stays in scalar registers
+    const auto ge = [wg](int e) { return (int)((uint32_t)(e - 1 - wg) >> 31); };
+    const int di = ge(e0) + ge(e1) + ge(e2) + ge(e3) + ge(e4) + ge(e5) + ge(e6) + ge(e7) + ge(e8) +
+                   ge(e9) + ge(e10) + ge(e11);
+    const Dot4GroupDesc d = tbl.d[di];
+    const GemvArgs a{d.A, d.B, d.out, d.s, d.ws, d.M, d.N, d.K, d.lpr_log2_passes & 0xff,
+                     d.lpr_log2_passes >> 8, pout_f32, d.div_magic};
+    gemv_dot4_body<BITS, MT, U, false, SF16>(a, wg - d.wg_begin, 0, pthreads, smem);
 }
 
 // ---------------------------------------------------------------------------

@@ -170,3 +170,70 @@ def test_grouped_graph_replay_and_argument_errors(oracle):
     A, B, s, ws = dev[0]
     with pytest.raises(RuntimeError):
         ops.packed_gemv_grouped([(A, B[:, :-32].contiguous(), s, ws)], bits=2)
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+def test_narrow_blocks_share_a_dot4_launch(oracle, bits):
+    """Blocks of one and two tokens go through the grouped form of the dot4 kernel: mixed widths,
+    ragged row counts, K from 128 to 9728 (rows shorter than the lanes that share them and rows
+    of many loads per lane), more problems than one launch holds."""
+    shapes = [(1, 2048, 2048), (2, 1024, 2048), (1, 2048, 6144), (2, 33, 128), (1, 1, 384),
+              (1, 1030, 2560), (2, 77, 9728), (1, 129, 4096), (2, 6144, 2048), (1, 17, 1536),
+              (1, 300, 640), (2, 255, 3072), (1, 64, 512), (2, 9, 1024)]
+    probs = [oracle.synth_problem(1100 + i, m, n, k, bits) for i, (m, n, k) in enumerate(shapes)]
+    check_group(oracle, probs, bits, "narrow")
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+@pytest.mark.parametrize("M", [1, 2])
+def test_narrow_grouped_equals_single_calls_bit_for_bit(oracle, bits, M):
+    """The grouped dot4 launch runs the body of the single-GEMV dot4 kernel: whatever lanes per
+    row and workgroup size the grouped launch picks, each row's lanes are added in the same tree
+    order only if the geometry matches, so the check forces one geometry for both calls."""
+    import bitmtp_amd as ops
+    from bitmtp_amd import ops as O2
+    lib = O2.t2_lib() if bits == 2 else O2.q1_lib()
+    set_tuning = lib.t2g128_set_tuning if bits == 2 else lib.q1g128_set_tuning
+    set_mfma = lib.t2g128_set_mfma_tuning if bits == 2 else lib.q1g128_set_mfma_tuning
+    probs = [oracle.synth_problem(1200 + i, M, n, k, bits) for i, (n, k) in enumerate(LAYER_17B)]
+    dev = [to_dev(p) for p in probs]
+    try:
+        set_tuning(16, 4, 0)
+        set_mfma(100, 0, 0, 0, 0)  # the single calls stay on the dot4 kernel at width 2 as well
+        grouped = ops.packed_gemv_grouped(dev, bits=bits, out_kind=ops.OUT_F32)
+        for i, (A, B, s, ws) in enumerate(dev):
+            alone = ops.packed_gemv_ex(A, B, s, ws, bits=bits, out_kind=ops.OUT_F32)
+            assert torch.equal(alone, grouped[i]), f"problem {i}"
+    finally:
+        set_tuning(0, 0, 0)
+        set_mfma(0, 0, 0, 0, 0)
+
+
+def test_narrow_grouped_fp16_scales_and_graph_replay(oracle):
+    import bitmtp_amd as ops
+    probs = [oracle.synth_problem(1300 + i, 1, n, k, 2) for i, (n, k) in enumerate(LAYER_17B)]
+    dev, ws16s = [], []
+    for p in probs:
+        A, B, s, _ = to_dev(p)
+        ws16 = oracle.bf16_bits_to_f32(p["ws"]).astype(np.float16)
+        ws16s.append(ws16)
+        dev.append((A, B, s, torch.from_numpy(ws16).to("cuda:0")))
+    y32 = ops.packed_gemv_grouped(dev, bits=2, out_kind=ops.OUT_F32)
+    for i, p in enumerate(probs):
+        ref, _ = oracle.c_gemv(p["A"], p["B"], p["s"], ws16s[i].view(np.uint16), 2, scale_is_f16=True)
+        got = y32[i].cpu().numpy()
+        assert np.all(np.abs(got - ref) <= ATOL + RTOL * np.abs(ref)), f"fp16 scales, problem {i}"
+    eager = [t.clone() for t in ops.packed_gemv_grouped(dev, bits=2)]
+    outs = [torch.empty_like(t) for t in eager]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        ops.packed_gemv_grouped(dev, bits=2, outs=outs)
+    for rep in range(3):
+        for t in outs:
+            t.zero_()
+        _ = ops.packed_gemv_grouped(dev, bits=2)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, eager):
+            assert torch.equal(a, b), f"replay {rep} differs"
