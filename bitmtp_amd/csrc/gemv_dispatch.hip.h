@@ -18,6 +18,7 @@
 #include "gemv_mfma.hip.h"
 #include "gemv_mx.hip.h"
 #include "gemv_mxs.hip.h"
+#include "gemv_rowreg.hip.h"
 #include "packed_gemv.hip.h"
 
 namespace bonsai {
@@ -332,6 +333,15 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     const MfmaTuning &mtu = mfma_tuning<BITS>();
     const int min_width = mtu.min_width > 0 ? mtu.min_width
                                             : (N >= kLongMatrixRows ? 2 : kDefaultMfmaMinWidth);
+    if constexpr (BITS == 2) {
+        if (mtu.engine == 6 || mtu.engine == 0) {
+            // one token against a very long matrix: activations in registers, v_dot8
+            const GemvProblem q{A, B, out, s, ws, M, N, K};
+            if (rowreg_problem_ok(q, out_kind, mtu.engine == 6))
+                return launch_rowreg(q, out_kind, scale_kind, st.n_cus[dev],
+                                     mxs_tuning<BITS>().wgs_per_cu, stream);
+        }
+    }
     if (mtu.engine == 5 || mtu.engine == 0) {
         // very long matrices: the streaming kernel, at every width up to 16
         const GemvProblem q{A, B, out, s, ws, M, N, K};

@@ -100,3 +100,91 @@ def test_stream_kernel_graph_replay(oracle):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep} differs"
+
+
+# ---- the single-token streaming kernel (activations in registers, v_dot8) -------------------
+@pytest.fixture
+def forced_rowreg():
+    from bitmtp_amd import ops as O2
+    t2 = O2.t2_lib()
+    t2.t2g128_set_mfma_tuning(0, 0, 0, 0, 6)
+    yield t2
+    t2.t2g128_set_mfma_tuning(0, 0, 0, 0, 0)
+    t2.t2g128_set_stream_tuning(0, 0)
+
+
+@pytest.mark.parametrize("N,K", [
+    (4096, 2048), (4099, 2048), (1, 2048), (7, 2048), (9, 1024), (1000, 1024), (33, 4096),
+    (5001, 4096), (40000, 2048), (20003, 1024),
+])
+def test_forced_single_token_kernel(oracle, forced_rowreg, N, K):
+    """8, 16 and 32 lanes per row (K = 1024, 2048, 4096); row counts that end inside a row
+    set, inside a batch, and matrices shorter than one batch of one wave."""
+    check_one(oracle, oracle.synth_problem(1600 + N, 1, N, K, 2), 2, "single token")
+
+
+@pytest.mark.parametrize("wgs_per_cu", [1, 2, 6])
+def test_forced_single_token_kernel_other_residency(oracle, forced_rowreg, wgs_per_cu):
+    forced_rowreg.t2g128_set_stream_tuning(0, wgs_per_cu)
+    check_one(oracle, oracle.synth_problem(1700 + wgs_per_cu, 1, 70001, 2048, 2), 2,
+              f"single token wgs/cu {wgs_per_cu}")
+
+
+def test_forced_single_token_kernel_extreme_bytes_and_fp16_scales(oracle, forced_rowreg):
+    """Every code value including 0 (-2), activations of -128 in every slot (the planes hold
+    hi = -8, lo = 0), fp16 group scales."""
+    import bitmtp_amd as ops
+    rng = np.random.default_rng(12)
+    p = oracle.synth_problem(1800, 1, 600, 2048, 2)
+    p["B"] = rng.integers(0, 256, size=p["B"].shape, dtype=np.uint8)
+    p["B"][0, :] = 0x00
+    p["B"][1, :] = 0xFF
+    for fill in (None, -128, 127):
+        p["A"] = rng.integers(-128, 128, size=p["A"].shape, dtype=np.int8)
+        if fill is not None:
+            p["A"][:] = fill
+        check_one(oracle, p, 2, f"extreme fill={fill}")
+        A, B, s, ws = to_dev(p)
+        G = ops.packed_gemv_ex(A, B, None, None, bits=2, out_kind=ops.OUT_G32)  # dot4 kernel: exact sums
+        assert np.array_equal(G.cpu().numpy(), oracle.c_group_sums(p["A"], p["B"], 2))
+    ws16 = oracle.bf16_bits_to_f32(p["ws"]).astype(np.float16)
+    A, B, s, _ = to_dev(p)
+    y32 = ops.packed_gemv_ex(A, B, s, torch.from_numpy(ws16).to("cuda:0"), bits=2,
+                             out_kind=ops.OUT_F32).cpu().numpy()
+    ref, _ = oracle.c_gemv(p["A"], p["B"], p["s"], ws16.view(np.uint16), 2, scale_is_f16=True)
+    assert np.all(np.abs(y32 - ref) <= ATOL + RTOL * np.abs(ref))
+
+
+def test_single_token_kernel_is_exact_for_unit_scales(oracle, forced_rowreg):
+    """With every group scale 1 and s = 1 the fp32 result is the integer dot product, exactly
+    (|sum| < 2^24): pins the plane arithmetic G = 16 H + L - 2 sum(a) bit for bit."""
+    import bitmtp_amd as ops
+    rng = np.random.default_rng(13)
+    N, K = 3000, 2048
+    A = rng.integers(-128, 128, size=(1, K), dtype=np.int8)
+    Bp = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    w = oracle.np_unpack(Bp, 2).astype(np.int64)
+    want = (w @ A[0].astype(np.int64)).astype(np.float32)
+    ws = torch.ones(N, K // 128, dtype=torch.bfloat16, device="cuda:0")
+    s = torch.ones(1, 1, dtype=torch.float32, device="cuda:0")
+    y = ops.packed_gemv_ex(torch.from_numpy(A).cuda(), torch.from_numpy(Bp.view(np.int8)).cuda(), s, ws,
+                           bits=2, out_kind=ops.OUT_F32).cpu().numpy()[0]
+    assert np.array_equal(y, want)
+
+
+def test_single_token_kernel_graph_replay(oracle):
+    import bitmtp_amd as ops
+    ops.init_kernels()
+    A, B, s, ws = to_dev(oracle.synth_problem(1900, 1, 151936, 2048, 2))
+    eager = ops.packed_gemv_ex(A, B, s, ws, bits=2).clone()
+    out = torch.empty_like(eager)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        ops.packed_gemv_ex(A, B, s, ws, bits=2, out=out)
+    for rep in range(3):
+        out.zero_()
+        _ = ops.packed_gemv_ex(A, B, s, ws, bits=2)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs"
