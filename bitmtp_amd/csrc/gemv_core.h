@@ -276,98 +276,5 @@ BONSAI_HD int mfma_stage_quarter(const u32x4 *src, u32x4 *act_token, int q) {
 template <int BITS>
 BONSAI_HD int mfma_corr(int group_asum) { return BITS == 2 ? -2 * group_asum : -group_asum; }
 
-// ---------------------------------------------------------------------------
-// FP4 x FP8 matrix-core path (v_mfma_f32_16x16x128_f8f6f4)
-// ---------------------------------------------------------------------------
-// One MFMA contracts a whole 128-weight group.  The weights go in as FP4 (E2M1),
-// whose codes 0..3 mean 0, 0.5, 1.0, 1.5 -- i.e. 0.5 * (T2 code) or 0.5 * (Q1 bit)
-// -- so "unpacking" is masking nibbles:
-//     T2: n0 = p0 & 0x33333333, n1 = (p0 >> 2) & 0x33333333, n2/n3 likewise from p1
-//         nibble i of n_v = weight 16*(v/2) + 2i + (v%2) of the lane's 32
-//     Q1: n_v = (p >> v) & 0x11111111, v = 0..3
-//         nibble i of n_v = weight 4i + v of the lane's 32
-// The activations go in as FP8 (E4M3) in two planes, 16*(a >> 4) and a & 15, both
-// exact in E4M3; two MFMAs accumulate 0.5 * sum a*code exactly in fp32 (every
-// partial sum is a multiple of 0.5 below 2^17).  The accumulator input carries
-// the offset removal, so the result is G/2 (T2) or G/4 (Q1) of the exact group
-// sum G.
-//
-// Operand slots, as measured on gfx950: lane (column j, K-block kb) of the FP4
-// operand holds K = 32*kb + n in nibble n (register n/8, low nibble first); lane
-// (row i, K-block kb) of the FP8 operand holds K = 16*kb + b in byte b < 16 and
-// K = 64 + 16*kb + (b - 16) in byte b >= 16.  Activations are therefore staged
-// per group and plane as 128 bytes in K order, H[32*q + n] = a[32*q + w(n)] with
-// w the nibble->weight map above, and a lane reads bytes 16kb..16kb+15 and
-// 64+16kb..64+16kb+15 of that block.
-template <int BITS>
-BONSAI_HD void fp4_unpack(uint32_t p0, uint32_t p1, uint32_t n[4]) {
-    if (BITS == 2) {
-        n[0] = p0 & 0x33333333u;
-        n[1] = (p0 >> 2) & 0x33333333u;
-        n[2] = p1 & 0x33333333u;
-        n[3] = (p1 >> 2) & 0x33333333u;
-    } else {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) n[v] = (p0 >> v) & 0x11111111u;
-    }
-}
-
-// Weight index (0..31 inside the lane's 32) held by nibble n of the FP4 operand.
-template <int BITS>
-BONSAI_HD int fp4_weight_of_nibble(int n) {
-    const int v = n >> 3, i = n & 7;
-    return BITS == 2 ? 16 * (v >> 1) + 2 * i + (v & 1) : 4 * i + v;
-}
-
-BONSAI_HD uint32_t pick4(uint32_t a, uint32_t b, uint32_t c, uint32_t d, int byte) {
-    return ((a >> (8 * byte)) & 0xffu) | (((b >> (8 * byte)) & 0xffu) << 8) |
-           (((c >> (8 * byte)) & 0xffu) << 16) | (((d >> (8 * byte)) & 0xffu) << 24);
-}
-
-// Reorders one 32-activation block (x[0..7], natural order) into operand K order:
-// byte n of the result = activation fp4_weight_of_nibble(n).
-template <int BITS>
-BONSAI_HD void fp4_order_block(const uint32_t x[8], uint32_t o[8]) {
-    if (BITS == 2) {
-        // per 16 activations: the eight even ones, then the eight odd ones
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const uint32_t a = x[4 * h], b = x[4 * h + 1], c = x[4 * h + 2], d = x[4 * h + 3];
-#if defined(__HIP_DEVICE_COMPILE__)
-            o[4 * h + 0] = __builtin_amdgcn_perm(b, a, 0x06040200u);  // a.b0 a.b2 b.b0 b.b2
-            o[4 * h + 1] = __builtin_amdgcn_perm(d, c, 0x06040200u);
-            o[4 * h + 2] = __builtin_amdgcn_perm(b, a, 0x07050301u);  // a.b1 a.b3 b.b1 b.b3
-            o[4 * h + 3] = __builtin_amdgcn_perm(d, c, 0x07050301u);
-#else
-            o[4 * h + 0] = (a & 0xffu) | (((a >> 16) & 0xffu) << 8) | ((b & 0xffu) << 16) |
-                           (((b >> 16) & 0xffu) << 24);
-            o[4 * h + 1] = (c & 0xffu) | (((c >> 16) & 0xffu) << 8) | ((d & 0xffu) << 16) |
-                           (((d >> 16) & 0xffu) << 24);
-            o[4 * h + 2] = ((a >> 8) & 0xffu) | ((a >> 24) << 8) | (((b >> 8) & 0xffu) << 16) |
-                           ((b >> 24) << 24);
-            o[4 * h + 3] = ((c >> 8) & 0xffu) | ((c >> 24) << 8) | (((d >> 8) & 0xffu) << 16) |
-                           ((d >> 24) << 24);
-#endif
-        }
-    } else {
-        // byte n = 8v + i  <-  activation 4i + v: byte v of dword i
-        const u32x4 t0 = transpose4x4_bytes(x[0], x[1], x[2], x[3]);  // t0.[v] = bytes v of x0..x3
-        const u32x4 t1 = transpose4x4_bytes(x[4], x[5], x[6], x[7]);
-        o[0] = t0.x; o[1] = t1.x;
-        o[2] = t0.y; o[3] = t1.y;
-        o[4] = t0.z; o[5] = t1.z;
-        o[6] = t0.w; o[7] = t1.w;
-    }
-}
-
-// Multiplier that turns the MFMA result into the exact group sum.
-template <int BITS>
-BONSAI_HD constexpr int fp4_result_scale() { return BITS == 2 ? 2 : 4; }
-// Accumulator input per (group, token): -asum (T2) or -asum/4 (Q1), exact in fp32.
-template <int BITS>
-BONSAI_HD float fp4_corr(int group_asum) {
-    return BITS == 2 ? -(float)group_asum : -0.25f * (float)group_asum;
-}
-
 }  // namespace bonsai
 #endif  // BONSAI_GEMV_CORE_H

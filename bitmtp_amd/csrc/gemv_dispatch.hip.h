@@ -4,17 +4,15 @@
 // on layer-sized matrices; from three tokens on (from two for very long matrices,
 // the lm_head) the int8 matrix-core kernels (gemv_mfma.hip.h) win: the one that
 // loads the activations straight as operands up to 16384 rows, the one that
-// stages them in LDS once per workgroup above.  The FP4 x FP8 matrix-core kernel
-// (gemv_fp4.hip.h) needs fewer VALU operations per byte but its FP8 staging and
-// deeper register use make it no faster yet; it runs only when selected with the
-// tuning call.  Shapes the matrix-core kernels do not take (K not a multiple of
+// stages them in LDS once per workgroup above; one token against a very long matrix
+// has a kernel of its own (gemv_rowreg.hip.h), wider blocks there take the streaming
+// matrix-core kernel (gemv_mxs.hip.h).  Shapes the matrix-core kernels do not take (K not a multiple of
 // 512, unaligned operands, token tiles that do not fit in LDS) go to the dot4
 // kernel.  Replaces the if-chain over registered (M, N, K) of the reference
 // (src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:94-148).
 #ifndef BONSAI_GEMV_DISPATCH_HIP_H
 #define BONSAI_GEMV_DISPATCH_HIP_H
 
-#include "gemv_fp4.hip.h"
 #include "gemv_mfma.hip.h"
 #include "gemv_mx.hip.h"
 #include "gemv_mxs.hip.h"
@@ -26,6 +24,16 @@ namespace bonsai {
 constexpr int kDefaultMfmaMinWidth = 3;       // layer-sized matrices (dot4 wins at 1 and 2 tokens)
 constexpr int kDirectMaxRows = 16384;         // up to here the staging-free matrix-core kernel
 constexpr int kLongMatrixRows = 32768;        // from here on the matrix cores pay off at M >= 2
+
+// Every kernel reads A and B with 16-byte vector loads and the scales as 16-bit words.
+inline bool operands_aligned(const void *A, const void *B, const void *out, const void *s,
+                             const void *ws, int out_kind) {
+    const auto mis = [](const void *p, uintptr_t a) {
+        return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0;
+    };
+    return !(mis(A, 16) || mis(B, 16) || mis(out, out_kind == OUT_BF16 ? 2 : 4) ||
+             (s != nullptr && mis(s, 4)) || (ws != nullptr && mis(ws, 2)));
+}
 
 // ---- grouped dot4 launch (narrow blocks) -------------------------------------------------
 constexpr int kDot4GroupMaxWidth = 2;  // widest block the grouped dot4 kernel takes
@@ -147,18 +155,19 @@ int launch_dot4_grouped(const GemvProblem *probs, int count, int out_kind, int s
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
+// One-time set-up of every kernel on the current device, under a lock: two host threads that
+// launch at the same moment initialise once.  The ready flag is written last.
 template <int BITS>
 int init_all_kernels() {
+    LibState<BITS> &st = lib_state<BITS>();
+    std::lock_guard<std::mutex> guard(st.init_mutex);
     const int rc = init_device<BITS>();
     if (rc != 0) return rc;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 2;
-    LibState<BITS> &st = lib_state<BITS>();
-    if (!st.mfma_ready[dev]) {
+    if (!st.mfma_ready[dev].load(std::memory_order_acquire)) {
         const int rc2 = mfma_init_device<BITS>(st.lds_limit[dev]);
         if (rc2 != 0) return rc2;
-        const int rc3 = fp4_init_device<BITS>(st.lds_limit[dev]);
-        if (rc3 != 0) return rc3;
         const int rc4 = mx_init_device<BITS>(st.lds_limit[dev]);
         if (rc4 != 0) return rc4;
         const int rc5 = mxs_init_device<BITS>(st.lds_limit[dev]);
@@ -170,12 +179,23 @@ int init_all_kernels() {
             cus <= 0)
             return 2;
         st.n_cus[dev] = cus;
-        st.mfma_ready[dev] = true;
+        st.mfma_ready[dev].store(true, std::memory_order_release);
     }
     return 0;
 }
 
-// Launches one of the matrix-core kernels (engine 1 staged int8, 2 FP4 x FP8, 3 direct int8).  Returns -1 when the shape does not
+// Set-up on first use.  A first launch on a capturing stream is refused (status 3) instead of
+// changing kernel attributes under capture: call *_init before capturing.
+template <int BITS>
+int ensure_ready(int dev, hipStream_t stream) {
+    LibState<BITS> &st = lib_state<BITS>();
+    if (st.mfma_ready[dev].load(std::memory_order_acquire)) return 0;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) return 3;
+    return init_all_kernels<BITS>();
+}
+
+// Launches one of the matrix-core kernels (engine 1 staged int8, 3 direct int8).  Returns -1 when the shape does not
 // fit (the caller falls back), 0 on success, 2 on a launch error.  `single_tile`
 // refuses shapes whose tokens would need more than ceil(M/16) token tiles, i.e.
 // a second pass over the weights.
@@ -184,11 +204,10 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
                        const float *s, const void *ws, int M, int N, int K, int out_kind,
                        int scale_kind, int lds_limit, hipStream_t stream) {
     const MfmaTuning &tu = mfma_tuning<BITS>();
-    const bool fp4 = engine == 2, direct = engine == 3;
+    const bool direct = engine == 3;
     int nw = 4;  // waves per workgroup; eight only for the direct kernel on long rows
     auto lds_for = [&](int ri, int mt) {
-        return fp4 ? fp4_lds_for<BITS>(ri, mt, K)
-                   : (direct ? mfma_direct_lds_for<BITS>(ri, nw) : mfma_lds_for<BITS>(ri, mt, K));
+        return direct ? mfma_direct_lds_for<BITS>(ri, nw) : mfma_lds_for<BITS>(ri, mt, K);
     };
     int ntok_tiles = (M + kMfmaTokens - 1) / kMfmaTokens;
     int mt = (M + ntok_tiles - 1) / ntok_tiles;
@@ -270,17 +289,16 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
     args.ks_log2 = flex ? ks : (ks == 8 ? 3 : (ks == 4 ? 2 : (ks == 2 ? 1 : 0)));
     args.out_f32 = out_kind == OUT_F32 ? 1 : 0;
     args.passes = passes;
-    const int per_token = fp4 ? K / 32 : K / mfma_quarter_bytes<BITS>();  // staging tasks per token
+    const int per_token = K / mfma_quarter_bytes<BITS>();  // staging tasks per token
     args.div_magic = (uint32_t)(0x100000000ull / (uint64_t)per_token) + 1u;
 
     const int rows_per_wg = 16 * R * (nw / ks) * passes;
     const int grid_x = (N + rows_per_wg - 1) / rows_per_wg;
     const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
-    const MfmaKernelFn fn = fp4 ? fp4_table<BITS>().fn[ri][variant]
-                                : (flex ? mfma_direct_flex_table<BITS>().fn[0][variant]
-                                   : direct ? (nw == 8 ? mfma_direct8_table<BITS>().fn[ri][variant]
-                                                       : mfma_direct_table<BITS>().fn[ri][variant])
-                                            : mfma_table<BITS>().fn[ri][variant]);
+    const MfmaKernelFn fn = flex ? mfma_direct_flex_table<BITS>().fn[0][variant]
+                            : direct ? (nw == 8 ? mfma_direct8_table<BITS>().fn[ri][variant]
+                                                : mfma_direct_table<BITS>().fn[ri][variant])
+                                     : mfma_table<BITS>().fn[ri][variant];
     hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(nw * 64, 1, 1), lds_for(ri, mt),
                        stream, args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
                        args.mt, args.ks_log2, args.out_f32, args.passes, args.div_magic);
@@ -320,12 +338,13 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     if (out_kind != OUT_G32 && (s == nullptr || ws == nullptr)) return 1;
     if (M < 1 || N < 1 || K < kGroup || K % kGroup != 0) return 1;
     if ((long)M * N > 0x7fffffffL / 2) return 1;  // row indices are 32-bit
+    if (!operands_aligned(A, B, out, s, ws, out_kind)) return 1;
 
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 2;
     LibState<BITS> &st = lib_state<BITS>();
-    if (st.lds_limit[dev] == 0 || !st.mfma_ready[dev]) {
-        const int rc = init_all_kernels<BITS>();
+    {
+        const int rc = ensure_ready<BITS>(dev, stream);
         if (rc != 0) return rc;
     }
     const int lds_limit = st.lds_limit[dev];
@@ -361,7 +380,7 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
         int rc = -1;
         // operand-loaded activations win up to about 16k rows, staged ones above (measured)
         const int engine = mtu.engine != 0 ? mtu.engine : (N <= kDirectMaxRows ? 3 : 1);
-        if (engine == 2 || engine == 3)
+        if (engine == 3)
             rc = launch_matrix_core<BITS>(engine, false, A, B, out, s, ws, M, N, K, out_kind,
                                           scale_kind, lds_limit, stream);
         if (rc < 0)
@@ -389,12 +408,13 @@ int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_
         if (out_kind != OUT_G32 && (q.s == nullptr || q.ws == nullptr)) return 1;
         if (q.M < 1 || q.N < 1 || q.K < kGroup || q.K % kGroup != 0) return 1;
         if ((long)q.M * q.N > 0x7fffffffL / 2) return 1;
+        if (!operands_aligned(q.A, q.B, q.out, q.s, q.ws, out_kind)) return 1;
     }
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 2;
     LibState<BITS> &st = lib_state<BITS>();
-    if (st.lds_limit[dev] == 0 || !st.mfma_ready[dev]) {
-        const int rc = init_all_kernels<BITS>();
+    {
+        const int rc = ensure_ready<BITS>(dev, stream);
         if (rc != 0) return rc;
     }
     const int lds_limit = st.lds_limit[dev];

@@ -565,7 +565,7 @@ struct MfmaTuning {
     int row_tiles = 0;   // R: 1, 2 or 4; 0 = heuristic
     int k_split = 0;     // waves along K: 1, 2, 4 (or 8: direct kernel, eight waves); 0 = heuristic
     int passes = 0;      // row blocks per workgroup; 0 = heuristic
-    int engine = 0;      // 0 = choose, 1 = int8 MFMA (staged), 2 = FP4 x FP8 MFMA, 3 = int8 MFMA (direct)
+    int engine = 0;      // 0 = choose, 1 = int8 MFMA (staged), 3 = int8 MFMA (direct), 4 = grouped kernel, 5 / 6 = streaming kernels
 };
 
 using MfmaKernelFn = void (*)(const int8_t *, const uint8_t *, void *, const float *,

@@ -23,6 +23,9 @@
 #define BONSAI_PACKED_GEMV_HIP_H
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <mutex>
 #include <stdint.h>
 #include <stdio.h>
 
@@ -397,7 +400,8 @@ template <int BITS>
 struct LibState {
     Tuning tuning;
     int lds_limit[kMaxDevices] = {};  // 0 = device not initialised yet
-    bool mfma_ready[kMaxDevices] = {};
+    std::atomic<bool> mfma_ready[kMaxDevices] = {};  // set last, under init_mutex
+    std::mutex init_mutex;
     int n_cus[kMaxDevices] = {};
 };
 

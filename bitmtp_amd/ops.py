@@ -217,9 +217,13 @@ def t2g128_int8xint2_linear(a_int8: torch.Tensor, b_packed: torch.Tensor, s: tor
     m, out_shape = _out_shape(a_int8, n, "t2g128")
     lib = t2_lib()
     out = torch.empty(*out_shape, dtype=torch.bfloat16, device=a_int8.device)
+    # the checked form of the same entry point: the drop-in symbol returns nothing, and a
+    # refused launch would hand back the uninitialised tensor
     with torch.cuda.device(a_int8.device):
-        lib.t2g128_int8xint2_linear(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws),
-                                    m, n, k, _stream(a_int8.device))
+        rc = lib.t2g128_gemv_ex(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws),
+                                m, n, k, OUT_BF16, SCALE_BF16, _stream(a_int8.device))
+    if rc != 0:
+        raise RuntimeError(f"t2g128: native launch failed with status {rc} (M={m}, N={n}, K={k})")
     return out
 
 
@@ -234,8 +238,10 @@ def q1g128_int8xint1_linear(a_int8: torch.Tensor, b_packed: torch.Tensor, s: tor
     lib = q1_lib()
     out = torch.empty(*out_shape, dtype=torch.bfloat16, device=a_int8.device)
     with torch.cuda.device(a_int8.device):
-        lib.q1g128_int8xint1_linear(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws),
-                                    m, n, k, _stream(a_int8.device))
+        rc = lib.q1g128_gemv_ex(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws),
+                                m, n, k, OUT_BF16, SCALE_BF16, _stream(a_int8.device))
+    if rc != 0:
+        raise RuntimeError(f"q1: native launch failed with status {rc} (M={m}, N={n}, K={k})")
     return out
 
 

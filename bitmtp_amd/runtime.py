@@ -20,10 +20,12 @@ Differences from the reference, by design:
 from __future__ import annotations
 
 import gc
+import time
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
+
 import torch
 
 from . import contracts, decode_ops, ops
@@ -336,8 +338,11 @@ class GraphAtlas:
             # the event after the replay: polling it returns sooner than a blocking
             # synchronisation wakes the thread up
             ev = g.io.uploaded
+            deadline = time.perf_counter() + 0.05
             while not ev.query():
-                pass
+                if time.perf_counter() > deadline:  # a replay is a millisecond: stop spinning
+                    ev.synchronize()
+                    break
         else:
             g.io.out_host.copy_(g.io.out, non_blocking=True)
             torch.cuda.current_stream(self.device).synchronize()

@@ -22,10 +22,10 @@
  *   C   bf16  [M, N]        C[m][n] = bf16( (sum_g fp32(G[m][n][g]) * ws[n][g]) / s[m] )
  *   G   int32 [M, N, K/128] exact group sums G[m][n][g] = sum_{k in g} A[m][k] * w[n][k]
  *
- * Preconditions: M >= 1, N >= 1, K >= 128 and K % 128 == 0, B rows 16-byte
- * aligned (true for every K % 128 == 0 when B itself is 16-byte aligned), A
- * 16-byte aligned.  Any M is accepted: widths above 8 are processed as several
- * token tiles inside one launch.
+ * Preconditions: M >= 1, N >= 1, K >= 128 and K % 128 == 0; A and B 16-byte
+ * aligned (every row then is, for K % 128 == 0), s 4-byte, ws 2-byte, C / out
+ * aligned to its element: anything else is refused with BONSAI_ERR_ARG.  Any M is
+ * accepted: wide blocks are processed as several token tiles.
  */
 #ifndef BONSAI_GEMV_H
 #define BONSAI_GEMV_H
@@ -38,8 +38,10 @@ extern "C" {
 
 /* Status codes of the int-returning entry points. */
 #define BONSAI_OK 0
-#define BONSAI_ERR_ARG 1    /* null pointer, M/N/K out of range, K % 128 != 0 */
+#define BONSAI_ERR_ARG 1    /* null pointer, M/N/K out of range, K % 128 != 0, misaligned operand */
 #define BONSAI_ERR_LAUNCH 2 /* hipLaunchKernel / attribute call failed */
+#define BONSAI_ERR_NOT_INIT 3 /* first launch on this device happened on a capturing stream:
+                                 call *_init before the capture */
 
 /* ---- drop-in entry points ------------------------------------------------ */
 

@@ -120,67 +120,3 @@ extern "C" int sim_group_sums_mfma(const int8_t *A, const uint8_t *B, int32_t *G
     if (bits == 2) run_mfma<2>(A, B, G, M, N, K); else run_mfma<1>(A, B, G, M, N, K);
     return 0;
 }
-
-// ---------------------------------------------------------------------------
-// FP4 x FP8 matrix-core path.  The MFMA is modelled by the slot pairing measured on
-// gfx950 (see gemv_core.h): FP4 lane kb, nibble n <-> K = 32kb + n; FP8 lane kb,
-// byte b <-> K = 16kb + b (b < 16) or 64 + 16kb + b - 16.  FP4 code c means 0.5*c;
-// the two FP8 planes add up to the int8 activation, so the model multiplies the
-// activation itself.  Checked: block ordering, nibble extraction, correction term.
-// ---------------------------------------------------------------------------
-template <int BITS>
-static void run_fp4(const int8_t *A, const uint8_t *B, int32_t *G, int M, int N, int K) {
-    const int ng = K / 128;
-    // staged activations in K order: H[tok][g][128]
-    std::vector<int8_t> H((size_t)M * K);
-    std::vector<float> corr((size_t)ng * M);
-    for (int tok = 0; tok < M; ++tok)
-        for (int g = 0; g < ng; ++g) {
-            int asum = 0;
-            for (int q = 0; q < 4; ++q) {
-                uint32_t x[8], o[8];
-                std::memcpy(x, A + (size_t)tok * K + g * 128 + q * 32, 32);
-                for (int i = 0; i < 8; ++i) asum += sum4_i8(x[i]);
-                fp4_order_block<BITS>(x, o);
-                std::memcpy(&H[(size_t)tok * K + g * 128 + q * 32], o, 32);
-            }
-            corr[(size_t)g * M + tok] = fp4_corr<BITS>(asum);
-        }
-    const int row_bytes = K * BITS / 8;
-    for (int n = 0; n < N; ++n)
-        for (int g = 0; g < ng; ++g)
-            for (int tok = 0; tok < M; ++tok) {
-                // FP4 operand of the four lanes kb: value per K
-                float wk[128];
-                for (int kb = 0; kb < 4; ++kb) {
-                    uint32_t p0, p1 = 0, nib[4];
-                    const uint8_t *grp = B + (size_t)n * row_bytes + (size_t)g * (128 * BITS / 8);
-                    if (BITS == 2) {
-                        std::memcpy(&p0, grp + kb * 8, 4);
-                        std::memcpy(&p1, grp + kb * 8 + 4, 4);
-                    } else {
-                        std::memcpy(&p0, grp + kb * 4, 4);
-                    }
-                    fp4_unpack<BITS>(p0, p1, nib);
-                    for (int nn = 0; nn < 32; ++nn)
-                        wk[32 * kb + nn] = 0.5f * (float)((nib[nn >> 3] >> (4 * (nn & 7))) & 0xf);
-                }
-                // FP8 operand of the four lanes kb: bytes 16kb.. and 64+16kb.. of the block
-                float d = corr[(size_t)g * M + tok];
-                const int8_t *blk = &H[(size_t)tok * K + g * 128];
-                for (int kb = 0; kb < 4; ++kb)
-                    for (int b = 0; b < 32; ++b) {
-                        const int k = b < 16 ? 16 * kb + b : 64 + 16 * kb + (b - 16);
-                        const int8_t aval = b < 16 ? blk[16 * kb + b] : blk[64 + 16 * kb + (b - 16)];
-                        d += (float)aval * wk[k];
-                    }
-                G[((size_t)tok * N + n) * ng + g] = (int32_t)(d * fp4_result_scale<BITS>());
-            }
-}
-
-extern "C" int sim_group_sums_fp4(const int8_t *A, const uint8_t *B, int32_t *G, int M, int N, int K,
-                                  int bits) {
-    if (K % 128 != 0) return 1;
-    if (bits == 2) run_fp4<2>(A, B, G, M, N, K); else run_fp4<1>(A, B, G, M, N, K);
-    return 0;
-}

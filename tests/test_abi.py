@@ -80,3 +80,27 @@ def test_decode_library_exports_and_binding(libs):
     # host-only query: partials are [M][heads][chunks][132] fp32
     assert decode_ops.attention_scratch_bytes(9, 16, 1024 + 17) == 9 * 16 * 17 * 132 * 4
     assert decode_ops.attention_scratch_bytes(0, 16, 64) == 0
+
+
+def test_argument_checks_need_no_gpu():
+    """The entry points refuse bad arguments before they touch the device: null pointers, a K
+    that is no multiple of 128, and operands that are not aligned for the 16-byte vector loads
+    (the pointers here are never dereferenced)."""
+    from bitmtp_amd import ops
+    t2, q1 = ops.t2_lib(), ops.q1_lib()
+    VP = ctypes.c_void_p
+    ok = dict(A=0x10000, B=0x20000, out=0x30000, s=0x40000, ws=0x50000)
+
+    def call(lib_fn, M=1, N=16, K=128, **over):
+        a = dict(ok, **over)
+        return lib_fn(VP(a["A"]), VP(a["B"]), VP(a["out"]), VP(a["s"]), VP(a["ws"]), M, N, K, 0, 0, None)
+
+    for fn in (t2.t2g128_gemv_ex, q1.q1g128_gemv_ex):
+        assert call(fn, A=None) == 1 and call(fn, B=None) == 1 and call(fn, out=None) == 1
+        assert call(fn, K=64) == 1 and call(fn, K=192) == 1 and call(fn, M=0) == 1 and call(fn, N=0) == 1
+        assert call(fn, A=0x10008) == 1 and call(fn, B=0x20004) == 1    # 16-byte loads
+        assert call(fn, ws=0x50001) == 1 and call(fn, s=0x40002) == 1 and call(fn, out=0x30001) == 1
+        assert call(fn, M=70000, N=151936) == 1                          # M * N beyond the index range
+    d = (ops.GemvDesc * 1)(ops.GemvDesc(0x10008, 0x20000, 0x30000, 0x40000, 0x50000, 1, 16, 2048, 0))
+    assert t2.t2g128_gemv_grouped(d, 1, 0, 0, None) == 1
+    assert t2.t2g128_gemv_grouped(d, 0, 0, 0, None) == 1
