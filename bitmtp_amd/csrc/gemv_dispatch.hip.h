@@ -15,6 +15,7 @@
 
 #include "gemv_mfma.hip.h"
 #include "gemv_mx.hip.h"
+#include "gemv_mxl.hip.h"
 #include "gemv_mxs.hip.h"
 #include "gemv_rowreg.hip.h"
 #include "packed_gemv.hip.h"
@@ -174,6 +175,8 @@ int init_all_kernels() {
         if (rc5 != 0) return rc5;
         const int rc6 = dot4_group_init_device<BITS>(st.lds_limit[dev]);
         if (rc6 != 0) return rc6;
+        const int rc7 = mxl_init_device<BITS>(st.lds_limit[dev]);
+        if (rc7 != 0) return rc7;
         int cus = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
             cus <= 0)
@@ -327,6 +330,16 @@ int launch_grouped_mx_only(const GemvProblem &q, int out_kind, int scale_kind, i
         sub.out = static_cast<unsigned char *>(q.out) + (size_t)m0 * per_tok * out_elt;
         batch[nb++] = sub;
     }
+    // the lean form where it applies (every token tile of at most 16, a layer-sized matrix)
+    const MxTuning &gtu = mx_tuning<BITS>();
+    if (out_kind != OUT_G32 && nb <= kMxlMaxDesc && gtu.row_tiles == 0 && gtu.max_wgs == 0) {
+        bool ok = true;
+        for (int i = 0; i < nb; ++i) ok = ok && mxl_problem_ok<BITS>(batch[i]);
+        if (ok) {
+            const int rc = launch_mxl<BITS>(batch, nb, out_kind, scale_kind, lds_limit, n_cus, stream);
+            if (rc != -1) return rc;
+        }
+    }
     return launch_mx<BITS>(batch, nb, out_kind, scale_kind, lds_limit, n_cus, stream);
 }
 
@@ -367,7 +380,14 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
         if (mxs_problem_ok<BITS>(q, out_kind, lds_limit, st.n_cus[dev], mtu.engine == 5))
             return launch_mxs<BITS>(q, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
     }
-    if (mtu.engine == 4 && M >= min_width) {
+    // Short rows (at most five K tiles, so at most two per wave) on layer-sized matrices: the
+    // lean grouped kernel with one descriptor.  Measured against the operand-loading kernel on the
+    // decode shapes of the 1.7B- and 4B-shaped models at widths 3-16: 8-15 % faster for K = 2048
+    // and 2560 (4096 x 2048 at nine tokens 3.53 against 3.78 us, 12288 x 2048 4.89 against 5.27);
+    // for K = 6144 and 9728 the one-slice-per-wave form of the operand-loading kernel stays ahead.
+    const bool lean_default = mtu.engine == 0 && M >= min_width && K <= 5 * kMxTileK &&
+                              N <= kLongMatrixRows && out_kind != OUT_G32;
+    if ((mtu.engine == 4 || lean_default) && M >= min_width) {
         // the grouped kernel with a single descriptor
         const GemvProblem q{A, B, out, s, ws, M, N, K};
         if (mx_problem_ok(q, out_kind == OUT_G32)) {
@@ -425,7 +445,16 @@ int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_
     int nb = 0;
     auto flush = [&]() -> int {
         if (nb == 0) return 0;
-        const int rc = launch_mx<BITS>(batch, nb, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
+        int rc = -1;
+        // the lean form where the launch is resident at once (tu.row_tiles or tu.max_wgs set:
+        // the striding kernel is being steered by hand)
+        if (nb <= kMxlMaxDesc && tu.row_tiles == 0 && tu.max_wgs == 0) {
+            bool ok = true;
+            for (int i = 0; i < nb; ++i) ok = ok && mxl_problem_ok<BITS>(batch[i]);
+            if (ok) rc = launch_mxl<BITS>(batch, nb, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
+        }
+        if (rc == -1)
+            rc = launch_mx<BITS>(batch, nb, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
         nb = 0;
         return rc;
     };
