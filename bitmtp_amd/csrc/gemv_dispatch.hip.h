@@ -385,8 +385,9 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     // decode shapes of the 1.7B- and 4B-shaped models at widths 3-16: 8-15 % faster for K = 2048
     // and 2560 (4096 x 2048 at nine tokens 3.53 against 3.78 us, 12288 x 2048 4.89 against 5.27);
     // for K = 6144 and 9728 the one-slice-per-wave form of the operand-loading kernel stays ahead.
-    const bool lean_default = mtu.engine == 0 && M >= min_width && K <= 5 * kMxTileK &&
-                              N <= kLongMatrixRows && out_kind != OUT_G32;
+    const bool lean_default = mtu.engine == 0 && M >= min_width && N <= kLongMatrixRows &&
+                              out_kind != OUT_G32 &&
+                              (K <= 5 * kMxTileK || (M <= kMfmaTokens && (N + 15) / 16 <= st.n_cus[dev]));
     if ((mtu.engine == 4 || lean_default) && M >= min_width) {
         // the grouped kernel with a single descriptor
         const GemvProblem q{A, B, out, s, ws, M, N, K};

@@ -58,13 +58,16 @@ __device__ __forceinline__ u32x4 mxl_load_b128(__amdgpu_buffer_rsrc_t rsrc, uint
 // LDS bytes of one workgroup: per wave the staged tokens of one K tile and one weight tile, then
 // the K-slice partials.
 template <int BITS>
-__host__ __device__ constexpr size_t mxl_lds_bytes(int mmax) {
-    return kMxWaves * mx_wave_lds_bytes<BITS, 1>(mmax) + (size_t)kMxWaves * 4 * 64 * 4;
+__host__ __device__ constexpr size_t mxl_lds_bytes(int mmax, int waves) {
+    return waves * mx_wave_lds_bytes<BITS, 1>(mmax) + (size_t)waves * 4 * 64 * 4;
 }
 
 // MR: result columns kept per lane (1 when every block of the launch has one token, else 4).
-template <int BITS, int MR, bool SF16>
-__global__ void __launch_bounds__(kMxThreads) __attribute__((amdgpu_waves_per_eu(4)))
+// W: waves per workgroup = K slices per row tile: four, or twelve for a single matrix with long
+// rows (K = 6144: one tile per wave instead of three in sequence, each of which would wait for its
+// own memory round trip).
+template <int BITS, int MR, bool SF16, int W>
+__global__ void __launch_bounds__(W * 64) __attribute__((amdgpu_waves_per_eu(W == 4 ? 4 : 3)))
 gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, int e8, int e9,
                 int e10, int e11, int out_f32, int mmax, const MxlTable tbl) {
     using MF = MfmaFmt<BITS>;
@@ -87,13 +90,13 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ld_row = lane / MF::kLanesPerRow, ld_col = lane % MF::kLanesPerRow;
     const int op_row = lane & 15, kb = lane >> 4;
-    const int tb = (KT * wave) >> 2, te = (KT * (wave + 1)) >> 2;  // never empty
+    const int tb = (KT * wave) / W, te = (KT * (wave + 1)) / W;  // empty for some waves when KT < W
 
     const uint32_t wave_bytes = (uint32_t)mx_wave_lds_bytes<BITS, 1>(mmax);
     unsigned char *wbase = smem + (uint32_t)wave * wave_bytes;
     u32x4 *act = reinterpret_cast<u32x4 *>(wbase);  // [mmax][33]
     unsigned char *wt = wbase + (uint32_t)mmax * (kMxTokenUnits * 16);
-    float *red = reinterpret_cast<float *>(smem + kMxWaves * wave_bytes);
+    float *red = reinterpret_cast<float *>(smem + W * wave_bytes);
 
     const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t *>(d.A), 0, M * K, kMxlBufferWord3);
@@ -156,8 +159,9 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
 
     // ---- prologue: activation loads (L2), then the weight tile (HBM), then the multiplier of
     // the token this lane will finish
-    ActRegs acur;
+    ActRegs acur, amore;  // tokens 0-7 and 8-15 of the tile
     act_load(acur, tb, 0);
+    if (nbatch > 1) act_load(amore, tb, 1);
     load_w(tb);
     float s_tok = 1.0f;
     if (wave < MR) {
@@ -178,11 +182,7 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
 
     for (int kt = tb; kt < te; ++kt) {
         act_store(acur, 0);
-        for (int b = 1; b < nbatch; ++b) {  // blocks of more than 8 tokens
-            ActRegs more;
-            act_load(more, kt, b);
-            act_store(more, b);
-        }
+        if (nbatch > 1) act_store(amore, 1);
 #pragma unroll
         for (int h = 0; h < MF::kLoads; ++h) {
             uint2 *d2 = reinterpret_cast<uint2 *>(park + h * MF::kRowsPerLoad * MF::kPitch);
@@ -192,6 +192,7 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
         const uint2 sc = scr;
         if (kt + 1 < te) {  // uniform: the next tile of this slice travels during the arithmetic
             act_load(acur, kt + 1, 0);
+            if (nbatch > 1) act_load(amore, kt + 1, 1);
             load_w(kt + 1);
         }
 #pragma unroll
@@ -226,13 +227,13 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
 
     // ---- K slices added in slice order; wave r finishes column r of every token quad
 #pragma unroll
-    for (int r = 0; r < MR; ++r) red[(r * kMxWaves + wave) * 64 + lane] = acc[r];
+    for (int r = 0; r < MR; ++r) red[(r * W + wave) * 64 + lane] = acc[r];
     __syncthreads();
     if (wave >= MR) return;
-    const float *mine = red + (wave * kMxWaves) * 64 + lane;
+    const float *mine = red + (wave * W) * 64 + lane;
     float y = mine[0];
 #pragma unroll
-    for (int k2 = 1; k2 < kMxWaves; ++k2) y += mine[k2 * 64];
+    for (int k2 = 1; k2 < W; ++k2) y += mine[k2 * 64];
     const int tk = 4 * kb + wave;
     const int row = n0 + op_row;
     if (row < N && tk < M) {
@@ -251,21 +252,29 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
 using MxlKernelFn = void (*)(int, int, int, int, int, int, int, int, int, int, int, int, int, int,
                              const MxlTable);
 
-template <int BITS>
-MxlKernelFn mxl_kernel(int scale_kind, bool one_token) {
+constexpr int kMxlWideWaves = 12;
+
+template <int BITS, int W>
+MxlKernelFn mxl_kernel_w(int scale_kind, bool one_token) {
     if (one_token)
-        return scale_kind == 1 ? gemv_mxl_kernel<BITS, 1, true> : gemv_mxl_kernel<BITS, 1, false>;
-    return scale_kind == 1 ? gemv_mxl_kernel<BITS, 4, true> : gemv_mxl_kernel<BITS, 4, false>;
+        return scale_kind == 1 ? gemv_mxl_kernel<BITS, 1, true, W> : gemv_mxl_kernel<BITS, 1, false, W>;
+    return scale_kind == 1 ? gemv_mxl_kernel<BITS, 4, true, W> : gemv_mxl_kernel<BITS, 4, false, W>;
+}
+template <int BITS>
+MxlKernelFn mxl_kernel(int scale_kind, bool one_token, bool wide) {
+    return wide ? mxl_kernel_w<BITS, kMxlWideWaves>(scale_kind, one_token)
+                : mxl_kernel_w<BITS, kMxWaves>(scale_kind, one_token);
 }
 
 template <int BITS>
 int mxl_init_device(int max_lds) {
     for (int sk = 0; sk < 2; ++sk)
         for (int one = 0; one < 2; ++one)
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(mxl_kernel<BITS>(sk, one != 0)),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    max_lds) != hipSuccess)
-                return 2;
+            for (int wide = 0; wide < 2; ++wide)
+                if (hipFuncSetAttribute(
+                        reinterpret_cast<const void *>(mxl_kernel<BITS>(sk, one != 0, wide != 0)),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, max_lds) != hipSuccess)
+                    return 2;
     return 0;
 }
 
@@ -291,7 +300,12 @@ int launch_mxl(const GemvProblem *probs, int count, int out_kind, int scale_kind
         mmax = probs[i].M > mmax ? probs[i].M : mmax;
         one_token = one_token && probs[i].M == 1;
     }
-    const size_t lds = mxl_lds_bytes<BITS>(mmax);
+    // twelve waves per workgroup: one matrix with rows of at least six K tiles whose workgroups
+    // find a CU each (the LDS of twelve staged tiles leaves one workgroup per CU)
+    const bool wide = count == 1 && probs[0].K >= 6 * kMxTileK && wgs <= n_cus &&
+                      mxl_lds_bytes<BITS>(mmax, kMxlWideWaves) <= (size_t)lds_limit;
+    const int waves = wide ? kMxlWideWaves : kMxWaves;
+    const size_t lds = mxl_lds_bytes<BITS>(mmax, waves);
     if (lds > (size_t)lds_limit) return -1;
     // layer-sized launches only: a few rounds of workgroups at most (longer matrices go to the
     // striding kernel, whose workgroups restage nothing they do not have to)
@@ -324,7 +338,7 @@ int launch_mxl(const GemvProblem *probs, int count, int out_kind, int scale_kind
         ends[i] = wg;
     }
     for (int i = count; i < kMxlMaxDesc; ++i) ends[i] = 0x7fffffff;
-    hipLaunchKernelGGL(mxl_kernel<BITS>(scale_kind, one_token), dim3(wg, 1, 1), dim3(kMxThreads, 1, 1),
+    hipLaunchKernelGGL(mxl_kernel<BITS>(scale_kind, one_token, wide), dim3(wg, 1, 1), dim3(waves * 64, 1, 1),
                        lds, stream, ends[0], ends[1], ends[2], ends[3], ends[4], ends[5], ends[6],
                        ends[7], ends[8], ends[9], ends[10], ends[11], out_kind == OUT_F32 ? 1 : 0,
                        mmax, tbl);
