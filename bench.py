@@ -381,8 +381,9 @@ def main() -> int:
         del g
     del mpool
 
-    # roofline of the dominant kernel: the grouped matrix-core kernel at the width whose
-    # launches take the most time; one launch streams one layer (13,369,344 algorithmic bytes)
+    # roofline of the dominant kernel: the grouped kernel at the width whose launches take the
+    # most time (one or two tokens: the grouped dot4 kernel, wider blocks: the lean grouped
+    # matrix-core kernel); one launch streams one layer (13,369,344 algorithmic bytes)
     dom = max(WIDTHS, key=lambda m: per_width[m]["us_per_launch"])
     bytes_per_launch = LAYER_BYTES
     achieved = bytes_per_launch / (per_width[dom]["us_per_launch"] * 1e-6) / 1e9
@@ -391,7 +392,8 @@ def main() -> int:
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "traffic": None if traffic is None else round(traffic),
-        "kernel": f"gemv_mx_kernel<BITS=2, R=1> (grouped, 7 descriptors, width {dom})",
+        "kernel": (f"gemv_dot4_grouped_kernel<BITS=2, MT={dom}>" if dom <= 2
+                   else "gemv_mxl_kernel<BITS=2, MR=4, W=4>") + f" (grouped, 7 descriptors, width {dom})",
         "bytes_per_launch": bytes_per_launch,
         "us_per_launch": per_width[dom]["us_per_launch"],
     }

@@ -59,7 +59,14 @@ def parse_shapes(text: str):
     return shapes
 
 
-def sweep(kind: str, shapes, widths, pool_bytes: int = 640 << 20, max_pool: int = 256, seed: int = 4):
+# --kernel: which kernel the single-GEMV entry point is steered to (development hooks of the
+# libraries); "auto" is the built-in choice
+KERNELS = {"auto": (0, 0), "dot4": (1000, 0), "staged": (1, 1), "operand": (1, 3), "lean": (1, 4),
+           "stream": (0, 5), "single-token": (0, 6)}
+
+
+def sweep(kind: str, shapes, widths, pool_bytes: int = 640 << 20, max_pool: int = 256, seed: int = 4,
+          kernel: str = "auto"):
     import torch
     import bitmtp_amd as ops
     from bitmtp_amd import ops as ops_mod
@@ -69,8 +76,10 @@ def sweep(kind: str, shapes, widths, pool_bytes: int = 640 << 20, max_pool: int 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     ops.init_kernels()
-    fn = (ops_mod.t2_lib().t2g128_int8xint2_linear if kind == "t2"
-          else ops_mod.q1_lib().q1g128_int8xint1_linear)
+    lib = ops_mod.t2_lib() if kind == "t2" else ops_mod.q1_lib()
+    fn = lib.t2g128_int8xint2_linear if kind == "t2" else lib.q1g128_int8xint1_linear
+    min_width, engine = KERNELS[kernel]
+    (lib.t2g128_set_mfma_tuning if kind == "t2" else lib.q1g128_set_mfma_tuning)(min_width, 0, 0, 0, engine)
     per_byte = 4 if kind == "t2" else 8
     gen = torch.Generator(device=dev)
     gen.manual_seed(seed)
@@ -119,7 +128,7 @@ def sweep(kind: str, shapes, widths, pool_bytes: int = 640 << 20, max_pool: int 
                 best = min(best, e0.elapsed_time(e1) * 1e-3 / count)
             del g
             results.append({
-                "kind": kind, "N": n, "K": k, "width": m, "bytes": nbytes, "pool": count,
+                "kind": kind, "kernel": kernel, "N": n, "K": k, "width": m, "bytes": nbytes, "pool": count,
                 "us_per_launch": round(best * 1e6, 3),
                 "gbps": round(nbytes / best / 1e9, 1),
                 "pct_hbm_peak": round(nbytes / best / 1e9 / HBM_PEAK_GBPS * 100, 2),
@@ -127,6 +136,7 @@ def sweep(kind: str, shapes, widths, pool_bytes: int = 640 << 20, max_pool: int 
             print(json.dumps(results[-1]), flush=True)
         del mats
         torch.cuda.empty_cache()
+    (lib.t2g128_set_mfma_tuning if kind == "t2" else lib.q1g128_set_mfma_tuning)(0, 0, 0, 0, 0)
     return results
 
 
@@ -137,12 +147,14 @@ def main() -> int:
     ap.add_argument("--shapes", default=None, help="comma list of NxK, e.g. 9728x2560,2560x9728")
     ap.add_argument("--widths", default="1,4,8", help="comma list and ranges, e.g. 1-8 or 1,4,8")
     ap.add_argument("--pool-mb", type=int, default=640, help="bytes of distinct matrices per shape")
+    ap.add_argument("--kernel", choices=sorted(KERNELS), default="auto",
+                    help="steer the entry point to one kernel (profiling runs)")
     args = ap.parse_args()
     if (args.preset is None) == (args.shapes is None):
         print("give exactly one of --preset and --shapes", file=sys.stderr)
         return 2
     shapes = PRESETS[args.preset] if args.preset else parse_shapes(args.shapes)
-    sweep(args.kind, shapes, parse_widths(args.widths), pool_bytes=args.pool_mb << 20)
+    sweep(args.kind, shapes, parse_widths(args.widths), pool_bytes=args.pool_mb << 20, kernel=args.kernel)
     return 0
 
 
