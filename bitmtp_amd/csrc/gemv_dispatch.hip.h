@@ -380,14 +380,15 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
         if (mxs_problem_ok<BITS>(q, out_kind, lds_limit, st.n_cus[dev], mtu.engine == 5))
             return launch_mxs<BITS>(q, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
     }
-    // Short rows (at most five K tiles, so at most two per wave) on layer-sized matrices: the
-    // lean grouped kernel with one descriptor.  Measured against the operand-loading kernel on the
-    // decode shapes of the 1.7B- and 4B-shaped models at widths 3-16: 8-15 % faster for K = 2048
-    // and 2560 (4096 x 2048 at nine tokens 3.53 against 3.78 us, 12288 x 2048 4.89 against 5.27);
-    // for K = 6144 and 9728 the one-slice-per-wave form of the operand-loading kernel stays ahead.
+    // Layer-sized matrices at three or more tokens: the lean grouped kernel with one descriptor per
+    // tile of up to 16 tokens, as long as its grid stays within eight workgroups per CU.  Measured
+    // against the operand-loading and the staged kernel at widths 3-16: 8-15 % faster on the
+    // K = 2048 / 2560 decode shapes of the 1.7B- and 4B-shaped models, 15-25 % on 12288 x 4096,
+    // 9728 x 9728, 24576 x 4096 and 27648 x 5120, level on 4096 x 12288 (where the twelve-wave
+    // form of the same kernel already ran).
+    const long lean_tiles = (long)((M + kMfmaTokens - 1) / kMfmaTokens) * ((N + 15) / 16);
     const bool lean_default = mtu.engine == 0 && M >= min_width && N <= kLongMatrixRows &&
-                              out_kind != OUT_G32 &&
-                              (K <= 5 * kMxTileK || (M <= kMfmaTokens && (N + 15) / 16 <= st.n_cus[dev]));
+                              out_kind != OUT_G32 && lean_tiles <= 8L * st.n_cus[dev];
     if ((mtu.engine == 4 || lean_default) && M >= min_width) {
         // the grouped kernel with a single descriptor
         const GemvProblem q{A, B, out, s, ws, M, N, K};
