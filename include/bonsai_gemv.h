@@ -174,12 +174,16 @@ int bonsai_silu_mul_quant_int8(const void *gate_up, int8_t *q, float *s, int M, 
  *   above any M disables them); 16-row tiles per wave (1, 2 or 4); waves of a workgroup that
  *   split K (1, 2, 4, 8, or 3..12 for the one-tile-per-wave form); row blocks a workgroup walks
  *   when K is not split; engine: 1 = int8 MFMA with activations staged in LDS, 3 = int8 MFMA
- *   with activations loaded as operands, 4 = the grouped kernel with one descriptor,
- *   5 = the streaming kernel on any shape it can run (otherwise only on very long matrices).
- * set_grouped_tuning: the grouped kernel -- 16-row tiles per wave (1 or 2), cap on the
- *   workgroups of one launch, smallest width sent to it.
- * set_stream_tuning: the streaming kernel for very long matrices -- smallest packed size in
- *   bytes that is sent to it (negative: never), persistent workgroups per CU. */
+ *   with activations loaded as operands, 4 = the grouped kernels with one descriptor (the lean
+ *   form where it applies), 5 = the streaming kernel on any shape it can run (otherwise only on
+ *   very long matrices), 6 = the single-token register kernel on any T2 matrix with K of 1024,
+ *   2048 or 4096 (otherwise only on very long ones).
+ * set_grouped_tuning: the grouped kernels -- 16-row tiles per wave (1 or 2) and a cap on the
+ *   workgroups of one launch (either one set selects the general grouped kernel instead of
+ *   its lean form), smallest width sent to the matrix cores (a value above zero also keeps
+ *   one- and two-token blocks off the grouped dot4 kernel).
+ * set_stream_tuning: the streaming kernels for very long matrices -- smallest packed size in
+ *   bytes that is sent to them (negative: never), persistent workgroups per CU. */
 void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
 void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes);
 void t2g128_set_mfma_tuning(int min_width, int row_tiles, int k_split, int passes, int engine);

@@ -3,7 +3,7 @@
 Only ``tests/`` and ``__graft_entry__.smoke()`` may import this module; the product
 (``bitmtp_amd``) never does.  NumPy only; bf16 values travel as uint16 bit patterns.
 
-What each function follows in the reference, and what pins it (tests/test_decode_oracle.py):
+What each function follows in the reference, and what pins it (tests/test_decode_host.py):
 
 * ``dense_mask_draft`` / ``dense_mask_causal``: the additive-mask templates and per-step
   patches of ``GraphAtlas`` (src/bonsai_sft/gpu/fast_runtime.py:316-372,391-465), as
