@@ -181,6 +181,31 @@ class Runner:
         return ts[0], ts[len(ts) // 2]
 
 
+
+def read_probe_us(torch, ops_mod, run, nbytes: int, workgroups: int, persistent: bool, dev) -> float:
+    """Microseconds per launch of the library's read probe (bonsai_read_probe: the same bytes
+    read once from HBM with the GEMV's launch shape and no arithmetic), timed like every other
+    figure here: one graph of launches over >= 512 MB of distinct buffers, best of 5 replays."""
+    probe = ops_mod.t2_lib().bonsai_read_probe
+    n = max(2, -(-MIN_DISTINCT_BYTES // nbytes))
+    bufs = torch.empty(n, nbytes, dtype=torch.uint8, device=dev).random_(0, 256)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = probe(bufs[0].data_ptr(), nbytes, workgroups, int(persistent), sink.data_ptr(), sp)
+    if rc != 0:
+        raise RuntimeError(f"bonsai_read_probe returned {rc}")
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        spc = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for i in range(n):
+            probe(bufs[i].data_ptr(), nbytes, workgroups, int(persistent), sink.data_ptr(), spc)
+    g.replay()
+    torch.cuda.synchronize()
+    t, _ = run.time_stats(g)
+    del g, bufs
+    return t / n * 1e6
+
 def cpu_baseline(budget_s: float):
     """Times the C oracle (OpenMP over output rows) on one layer at widths 1, 4, 8 --
     the same 21 GEMVs as one step -- repeating it until about `budget_s` seconds."""
@@ -327,6 +352,13 @@ def main() -> int:
         return table
 
     per_width = width_table(grouped=True)          # 1 launch per layer and width
+    # what the machine needs for the bytes of one layer alone: 1280 workgroups (one per 16 rows,
+    # as the grouped launch), every thread's loads requested up front
+    probe_layer_us = read_probe_us(torch, ops_mod, run, LAYER_BYTES, sum(n for _, n, _ in PROJECTIONS) // 16,
+                                   False, dev)
+    for m in WIDTHS:
+        per_width[m]["read_probe_us"] = round(probe_layer_us, 3)
+        per_width[m]["pct_of_read_probe"] = round(probe_layer_us / per_width[m]["us_per_launch"] * 100, 1)
     skip_drop_in = args.no_drop_in
     per_width_dropin = {} if skip_drop_in else width_table(grouped=False)  # 7 launches per layer
 
@@ -396,6 +428,7 @@ def main() -> int:
                    else "gemv_mxl_kernel<BITS=2, MR=4, W=4>") + f" (grouped, 7 descriptors, width {dom})",
         "bytes_per_launch": bytes_per_launch,
         "us_per_launch": per_width[dom]["us_per_launch"],
+        "read_probe_us": per_width[dom]["read_probe_us"],
     }
 
     # The one bandwidth-bound GEMV of the model, for scale: the packed lm_head
@@ -421,6 +454,12 @@ def main() -> int:
                             "pct_hbm_peak": round(hbytes / t / 1e9 / HBM_PEAK_GBPS * 100, 1)}
             del g
         del hpool
+        # the same bytes with no arithmetic, persistent workgroups as the head kernels launch them
+        props = torch.cuda.get_device_properties(dev)
+        probe_head_us = read_probe_us(torch, ops_mod, run, hbytes, 2 * props.multi_processor_count, True, dev)
+        for m in WIDTHS:
+            head[str(m)]["read_probe_us"] = round(probe_head_us, 2)
+            head[str(m)]["pct_of_read_probe"] = round(probe_head_us / head[str(m)]["us_per_launch"] * 100, 1)
 
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)

@@ -363,8 +363,11 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     const int lds_limit = st.lds_limit[dev];
 
     const MfmaTuning &mtu = mfma_tuning<BITS>();
+    // two tokens go to the matrix cores for very long matrices and for long rows (K >= 4096: at
+    // two tokens 2048 x 6144 takes 3.74 us there against 4.23 us on the dot4 kernel, 2560 x 9728
+    // 4.77 against 5.91; K = 2048 and 2560 are level or slower)
     const int min_width = mtu.min_width > 0 ? mtu.min_width
-                                            : (N >= kLongMatrixRows ? 2 : kDefaultMfmaMinWidth);
+                                            : (N >= kLongMatrixRows || K >= 4096 ? 2 : kDefaultMfmaMinWidth);
     if constexpr (BITS == 2) {
         if (mtu.engine == 6 || mtu.engine == 0) {
             // one token against a very long matrix: activations in registers, v_dot8

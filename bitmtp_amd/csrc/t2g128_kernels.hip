@@ -2,6 +2,7 @@
 // gfx950.  Entry points are declared in include/bonsai_gemv.h; the drop-in one
 // replaces src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:123-148.
 #include "gemv_dispatch.hip.h"
+#include "read_probe.hip.h"
 
 #include "../../include/bonsai_gemv.h"
 
@@ -42,6 +43,11 @@ void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width) {
     t.row_tiles = row_tiles;
     t.max_wgs = max_wgs;
     t.min_width = min_width;
+}
+
+int bonsai_read_probe(const void *src, size_t bytes, int workgroups, int persistent, void *sink,
+                      void *stream) {
+    return launch_read_probe(src, bytes, workgroups, persistent, sink, static_cast<hipStream_t>(stream));
 }
 
 void t2g128_set_stream_tuning(int min_bytes, int wgs_per_cu) {

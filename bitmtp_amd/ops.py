@@ -91,6 +91,9 @@ def load_t2_kernel() -> None:
     lib.t2g128_set_grouped_tuning.restype = None
     lib.t2g128_set_stream_tuning.argtypes = [ctypes.c_int] * 2
     lib.t2g128_set_stream_tuning.restype = None
+    lib.bonsai_read_probe.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_void_p, ctypes.c_void_p]
+    lib.bonsai_read_probe.restype = ctypes.c_int
     _t2_lib = lib
 
 

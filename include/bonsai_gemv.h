@@ -30,6 +30,7 @@
 #ifndef BONSAI_GEMV_H
 #define BONSAI_GEMV_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -192,6 +193,17 @@ void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
 void q1g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
 void t2g128_set_stream_tuning(int min_bytes, int wgs_per_cu);
 void q1g128_set_stream_tuning(int min_bytes, int wgs_per_cu);
+
+/* Measurement aid (libbonsai_t2.so; no reference counterpart, no arithmetic): reads `bytes` of
+ * device memory at `src` (16-byte aligned) exactly once with `workgroups` workgroups of 256
+ * threads and discards them.  persistent = 0: every thread requests its share up front (at most
+ * eight 16-byte loads, else BONSAI_ERR_ARG) -- the launch shape of a layer-sized GEMV;
+ * persistent = 1: workgroups loop with eight loads per lane in flight -- the shape of the
+ * kernels for very long matrices.  `sink` is 4 writable device bytes (practically never
+ * written).  bench.py times it beside the GEMV on the same byte counts: what the machine
+ * needs for the bytes alone. */
+int bonsai_read_probe(const void *src, size_t bytes, int workgroups, int persistent, void *sink,
+                      void *stream);
 
 #ifdef __cplusplus
 }

@@ -104,3 +104,11 @@ def test_argument_checks_need_no_gpu():
     d = (ops.GemvDesc * 1)(ops.GemvDesc(0x10008, 0x20000, 0x30000, 0x40000, 0x50000, 1, 16, 2048, 0))
     assert t2.t2g128_gemv_grouped(d, 1, 0, 0, None) == 1
     assert t2.t2g128_gemv_grouped(d, 0, 0, 0, None) == 1
+    # the read probe: null or misaligned pointers, and a one-shot launch of more than eight loads
+    # per thread (256 threads x 16 bytes x 8 per workgroup)
+    probe = t2.bonsai_read_probe
+    assert probe(None, 4096, 1, 0, VP(0x40000), None) == 1
+    assert probe(VP(0x10000), 4096, 1, 0, None, None) == 1
+    assert probe(VP(0x10008), 4096, 1, 0, VP(0x40000), None) == 1
+    assert probe(VP(0x10000), 4096, 0, 0, VP(0x40000), None) == 1
+    assert probe(VP(0x10000), 256 * 16 * 8 + 16, 1, 0, VP(0x40000), None) == 1

@@ -188,3 +188,20 @@ def test_single_token_kernel_graph_replay(oracle):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep} differs"
+
+
+@pytest.mark.parametrize("persistent", [0, 1])
+@pytest.mark.parametrize("nbytes, workgroups", [(16, 1), (4096 * 3 + 16, 2), (1 << 20, 64), (13369344, 1280)])
+def test_read_probe_runs_and_writes_nothing(nbytes, workgroups, persistent):
+    """The measurement aid reads its buffer (including a ragged tail) and leaves the sink and the
+    buffer as they were."""
+    import ctypes
+    from bitmtp_amd import ops
+    buf = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+    before = buf.clone()
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = ops.t2_lib().bonsai_read_probe(buf.data_ptr(), nbytes, workgroups, persistent, sink.data_ptr(), sp)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert int(sink.item()) == 0 and torch.equal(buf, before)
