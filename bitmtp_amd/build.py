@@ -1,4 +1,5 @@
-"""Builds the gfx950 shared libraries of this package with hipcc, in-tree.
+"""Builds the gfx950 shared libraries of this package with hipcc, in-tree, and the PyTorch
+operator library on top of them with g++.
 
     python -m bitmtp_amd.build            # build what is missing or out of date
     python -m bitmtp_amd.build --force    # rebuild everything
@@ -78,5 +79,43 @@ def build_all(force: bool = False, verbose: bool = True) -> list[str]:
     return [lib_path(s) for s in TARGETS if os.path.exists(lib_path(s))]
 
 
+# ---- the PyTorch operator library (host code only, g++) ---------------------------------
+TORCH_OPS_SOURCE = "torch_ops.cpp"
+TORCH_OPS_LIB = os.path.join("torch_ops", "libbonsai_torch.so")
+
+
+def torch_ops_path() -> str:
+    return os.path.join(HERE, TORCH_OPS_LIB)
+
+
+def build_torch_ops(force: bool = False, verbose: bool = True) -> str:
+    """Compiles csrc/torch_ops.cpp against the installed PyTorch and links it to the three C-ABI
+    libraries it calls (found at run time next to it through $ORIGIN).  No device code."""
+    out = torch_ops_path()
+    if not force and not _stale(out):
+        return out
+    build_all(verbose=verbose)  # the libraries it links to
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    libdirs = [os.path.dirname(lib_path(s)) for s in ("t2g128_kernels.hip", "q1g128_kernels.hip", "act_quant.hip")]
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f"-I{tdir}/include", f"-I{tdir}/include/torch/csrc/api/include", f"-I{rocm}/include",
+           os.path.join(CSRC, TORCH_OPS_SOURCE), "-o", out,
+           f"-L{tdir}/lib", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip"]
+    cmd += [f"-L{d}" for d in libdirs] + ["-lbonsai_t2", "-lbonsai_q1", "-lbonsai_actq",
+            "-Wl,-rpath,$ORIGIN/../t2g128_kernels:$ORIGIN/../q1g128_kernels:$ORIGIN/../act_quant"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"g++ failed for {TORCH_OPS_SOURCE}:\n{proc.stdout}")
+    if verbose:
+        print(f"[bitmtp_amd.build] built {os.path.relpath(out, HERE)}")
+    return out
+
+
 if __name__ == "__main__":
     build_all(force="--force" in sys.argv[1:])
+    build_torch_ops(force="--force" in sys.argv[1:])

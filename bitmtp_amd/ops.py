@@ -145,6 +145,30 @@ def load_actq_kernel() -> None:
     _actq_lib = lib
 
 
+_torch_ops_loaded = False
+
+
+def torch_ops_lib_path() -> str:
+    return os.path.join(_HERE, "torch_ops", "libbonsai_torch.so")
+
+
+def load_torch_ops():
+    """Registers the dispatcher operators ``torch.ops.bonsai.t2g128_int8xint2_linear``,
+    ``q1g128_int8xint1_linear`` and ``quant_input`` (CUDA and Meta kernels; csrc/torch_ops.cpp)
+    and returns the ``torch.ops.bonsai`` namespace.  Same tensors in and out as the functions of
+    this module (reference: model.py:118-268,632-636); a missing library raises."""
+    global _torch_ops_loaded
+    if not _torch_ops_loaded:
+        so = torch_ops_lib_path()
+        if not os.path.exists(so):
+            raise RuntimeError(
+                f"{so} is missing: build it with `python -m bitmtp_amd.build` "
+                "(there is no fallback implementation)")
+        torch.ops.load_library(so)
+        _torch_ops_loaded = True
+    return torch.ops.bonsai
+
+
 def t2_lib() -> ctypes.CDLL:
     if _t2_lib is None:
         load_t2_kernel()
