@@ -66,8 +66,15 @@ __host__ __device__ constexpr size_t mxl_lds_bytes(int mmax, int waves) {
 // W: waves per workgroup = K slices per row tile: four, or twelve for a single matrix with long
 // rows (K = 6144: one tile per wave instead of three in sequence, each of which would wait for its
 // own memory round trip).
-template <int BITS, int MR, bool SF16, int W>
-__global__ void __launch_bounds__(W * 64) __attribute__((amdgpu_waves_per_eu(W == 4 ? 4 : 3)))
+// NB: token batches of eight a block can have (2 only when some block has more than eight tokens):
+// without the registers of a second batch the four-wave form fits five waves per SIMD, so the
+// 1280 workgroups of a layer-sized launch are all resident at once instead of 1024 of them.
+// OCC: waves per SIMD the register allocation aims at.  With two batches five waves fit only
+// at exactly 96 registers, which costs about 0.1 us on launches that have no fifth workgroup per
+// CU to place, and saves a microsecond on those that do (19456 x 2560 at nine tokens 8.6 ->
+// 7.6 us), so the host picks per launch.
+template <int BITS, int MR, bool SF16, int W, int NB, int OCC>
+__global__ void __launch_bounds__(W * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, int e8, int e9,
                 int e10, int e11, int out_f32, int mmax, const MxlTable tbl) {
     using MF = MfmaFmt<BITS>;
@@ -159,9 +166,9 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
 
     // ---- prologue: activation loads (L2), then the weight tile (HBM), then the multiplier of
     // the token this lane will finish
-    ActRegs acur, amore;  // tokens 0-7 and 8-15 of the tile
+    ActRegs acur, amore;  // tokens 0-7 and 8-15 of the tile (amore unused when NB == 1)
     act_load(acur, tb, 0);
-    if (nbatch > 1) act_load(amore, tb, 1);
+    if (NB > 1 && nbatch > 1) act_load(amore, tb, 1);
     load_w(tb);
     float s_tok = 1.0f;
     if (wave < MR) {
@@ -182,7 +189,7 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
 
     for (int kt = tb; kt < te; ++kt) {
         act_store(acur, 0);
-        if (nbatch > 1) act_store(amore, 1);
+        if (NB > 1 && nbatch > 1) act_store(amore, 1);
 #pragma unroll
         for (int h = 0; h < MF::kLoads; ++h) {
             uint2 *d2 = reinterpret_cast<uint2 *>(park + h * MF::kRowsPerLoad * MF::kPitch);
@@ -192,7 +199,7 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
         const uint2 sc = scr;
         if (kt + 1 < te) {  // uniform: the next tile of this slice travels during the arithmetic
             act_load(acur, kt + 1, 0);
-            if (nbatch > 1) act_load(amore, kt + 1, 1);
+            if (NB > 1 && nbatch > 1) act_load(amore, kt + 1, 1);
             load_w(kt + 1);
         }
 #pragma unroll
@@ -254,27 +261,33 @@ using MxlKernelFn = void (*)(int, int, int, int, int, int, int, int, int, int, i
 
 constexpr int kMxlWideWaves = 12;
 
-template <int BITS, int W>
-MxlKernelFn mxl_kernel_w(int scale_kind, bool one_token) {
-    if (one_token)
-        return scale_kind == 1 ? gemv_mxl_kernel<BITS, 1, true, W> : gemv_mxl_kernel<BITS, 1, false, W>;
-    return scale_kind == 1 ? gemv_mxl_kernel<BITS, 4, true, W> : gemv_mxl_kernel<BITS, 4, false, W>;
+// width class: 0 = every block has one token, 1 = at most eight tokens, 2 = up to sixteen;
+// dense: more than four workgroups per CU to place (only matters for width class 2)
+template <int BITS, int W, int OCC1, int OCC2>
+MxlKernelFn mxl_kernel_w(int scale_kind, int width_class) {
+    if (width_class == 0)
+        return scale_kind == 1 ? gemv_mxl_kernel<BITS, 1, true, W, 1, OCC1> : gemv_mxl_kernel<BITS, 1, false, W, 1, OCC1>;
+    if (width_class == 1)
+        return scale_kind == 1 ? gemv_mxl_kernel<BITS, 4, true, W, 1, OCC1> : gemv_mxl_kernel<BITS, 4, false, W, 1, OCC1>;
+    return scale_kind == 1 ? gemv_mxl_kernel<BITS, 4, true, W, 2, OCC2> : gemv_mxl_kernel<BITS, 4, false, W, 2, OCC2>;
 }
 template <int BITS>
-MxlKernelFn mxl_kernel(int scale_kind, bool one_token, bool wide) {
-    return wide ? mxl_kernel_w<BITS, kMxlWideWaves>(scale_kind, one_token)
-                : mxl_kernel_w<BITS, kMxWaves>(scale_kind, one_token);
+MxlKernelFn mxl_kernel(int scale_kind, int width_class, bool wide, bool dense) {
+    if (wide) return mxl_kernel_w<BITS, kMxlWideWaves, 3, 3>(scale_kind, width_class);
+    return dense ? mxl_kernel_w<BITS, kMxWaves, 5, 5>(scale_kind, width_class)
+                 : mxl_kernel_w<BITS, kMxWaves, 5, 4>(scale_kind, width_class);
 }
 
 template <int BITS>
 int mxl_init_device(int max_lds) {
     for (int sk = 0; sk < 2; ++sk)
-        for (int one = 0; one < 2; ++one)
+        for (int wc = 0; wc < 3; ++wc)
             for (int wide = 0; wide < 2; ++wide)
-                if (hipFuncSetAttribute(
-                        reinterpret_cast<const void *>(mxl_kernel<BITS>(sk, one != 0, wide != 0)),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, max_lds) != hipSuccess)
-                    return 2;
+                for (int dense = 0; dense < 2; ++dense)
+                    if (hipFuncSetAttribute(
+                            reinterpret_cast<const void *>(mxl_kernel<BITS>(sk, wc, wide != 0, dense != 0)),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, max_lds) != hipSuccess)
+                        return 2;
     return 0;
 }
 
@@ -319,6 +332,8 @@ int launch_mxl(const GemvProblem *probs, int count, int out_kind, int scale_kind
             order[j] = order[j - 1];
             order[j - 1] = t;
         }
+    // a fifth workgroup per CU: only when the launch has one to place and the LDS holds it
+    const bool dense = !wide && wgs > 4L * n_cus && 5 * lds <= (size_t)lds_limit;
     MxlTable tbl{};
     int ends[kMxlMaxDesc];
     int wg = 0;
@@ -338,7 +353,7 @@ int launch_mxl(const GemvProblem *probs, int count, int out_kind, int scale_kind
         ends[i] = wg;
     }
     for (int i = count; i < kMxlMaxDesc; ++i) ends[i] = 0x7fffffff;
-    hipLaunchKernelGGL(mxl_kernel<BITS>(scale_kind, one_token, wide), dim3(wg, 1, 1), dim3(waves * 64, 1, 1),
+    hipLaunchKernelGGL(mxl_kernel<BITS>(scale_kind, one_token ? 0 : (mmax <= 8 ? 1 : 2), wide, dense), dim3(wg, 1, 1), dim3(waves * 64, 1, 1),
                        lds, stream, ends[0], ends[1], ends[2], ends[3], ends[4], ends[5], ends[6],
                        ends[7], ends[8], ends[9], ends[10], ends[11], out_kind == OUT_F32 ? 1 : 0,
                        mmax, tbl);

@@ -508,6 +508,8 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
     const bool pair_odd = BITS == 2 && g.mt == 1 && it >= 3;
     g.batch_index = (it % 4 == 0 || it >= 8) ? 2 : ((it % 2 == 0 || pair_odd) ? 1 : 0);
     if (g.batch_index > max_batch_index(g.mt)) g.batch_index = max_batch_index(g.mt);
+    // (1-bit chunks unpack to twice the registers: four loads per batch spill from two tokens on)
+    if (BITS == 1 && g.mt >= 2 && g.batch_index > 1) g.batch_index = 1;
     const int rpw = 64 >> g.lpr_log2;
     const long wave_passes = ((long)N + rpw - 1) / rpw;
 
