@@ -318,11 +318,13 @@ MxsTuning &mxs_tuning() {
     return t;
 }
 
-// Persistent workgroups per CU: four, fewer when the staged activations are large.
+// Persistent workgroups per CU: three (measured on the 151936 x 2048 head at 4 / 8 / 9 / 16 tokens:
+// 21.1 / 21.5 / 21.6 / 23.4 us against 21.9 / 22.5 / 22.1 / 22.9 us with four and no better with
+// five to eight), fewer when the staged activations are large.
 template <int BITS>
 int mxs_wgs_per_cu(const GemvProblem &q, int lds_limit) {
     const MxsTuning &tu = mxs_tuning<BITS>();
-    int per_cu = tu.wgs_per_cu > 0 ? tu.wgs_per_cu : 4;
+    int per_cu = tu.wgs_per_cu > 0 ? tu.wgs_per_cu : 3;
     const int fit = (int)((size_t)lds_limit / mxs_lds_bytes<BITS>(q.M, q.K));
     return per_cu < fit ? per_cu : fit;
 }
