@@ -61,8 +61,8 @@ const Dot4GroupKernels<BITS> &dot4_group_kernels() {
         x.fn[1][0][1] = gemv_dot4_grouped_kernel<BITS, 2, 1, true>;
         x.fn[1][1][0] = gemv_dot4_grouped_kernel<BITS, 2, 2, false>;
         x.fn[1][1][1] = gemv_dot4_grouped_kernel<BITS, 2, 2, true>;
-        x.fn[1][2][0] = gemv_dot4_grouped_kernel<BITS, 2, 4, false>;
-        x.fn[1][2][1] = gemv_dot4_grouped_kernel<BITS, 2, 4, true>;
+        x.fn[1][2][0] = gemv_dot4_grouped_kernel<BITS, 2, 2, false>;  // (never picked: two tokens take
+        x.fn[1][2][1] = gemv_dot4_grouped_kernel<BITS, 2, 2, true>;   //  at most two loads per batch)
         return x;
     }();
     return t;
@@ -106,9 +106,11 @@ int launch_dot4_grouped(const GemvProblem *probs, int count, int out_kind, int s
     int waves = 8, batch_index = kBatchKinds - 1;
     size_t lds = 0;
     // A launch of several matrices has waves enough without spreading every row over many
-    // lanes: at most sixteen lanes per row with at least two loads each, four waves per
-    // workgroup (sweep over the seven projections of the 1.7B-shaped layer, one token:
-    // 5.65 us against 6.4 us with each matrix's own single-launch geometry).
+    // lanes: eight lanes per row (four for 1-bit rows), sixteen once that leaves a lane eight
+    // chunks or more, four waves per workgroup.  Sweeps over the seven projections of a layer at
+    // one token: 1.7B-shaped 5.04 us (8 lanes for K = 2048, 16 for K = 6144) against 5.4 us with
+    // 16 / 16, 5.2-5.3 us with 16 / 32 or 16 / 64 and 6.4 us with each matrix's own
+    // single-launch geometry; 4B-shaped 8.4 against 8.8 us, Q1 7.3 against 7.4 us.
     Tuning tu = lib_state<BITS>().tuning;
     const bool own_rule = tu.lanes_per_row == 0 && tu.waves_per_wg == 0 && count > 1;
     for (int i = 0; i < count; ++i) {
@@ -117,7 +119,7 @@ int launch_dot4_grouped(const GemvProblem *probs, int count, int out_kind, int s
         if (own_rule) {
             const int C = q.K / Fmt<BITS>::kChunkWeights;
             int lpr = BITS == 1 ? 4 : 8;
-            while (lpr < 16 && 2 * lpr * 2 <= C) lpr *= 2;
+            while (lpr < 16 && 4 * lpr * 2 <= C) lpr *= 2;
             t.lanes_per_row = lpr;
             t.waves_per_wg = 4;
         }

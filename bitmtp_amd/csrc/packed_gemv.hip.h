@@ -366,9 +366,11 @@ void fill_table_cell(KernelTable<BITS> &t) {
 }
 
 // Register use grows with MT*U (the compiler keeps a whole batch unpacked), so
-// wide token tiles get shorter batches: U <= 4 for MT <= 2, U <= 2 for MT <= 4,
-// U = 1 above.  Cells that are not instantiated stay null.
-constexpr int max_batch_index(int mt) { return mt <= 2 ? 2 : (mt <= 4 ? 1 : 0); }
+// wide token tiles get shorter batches: U <= 4 for one token, U <= 2 for MT <= 4,
+// U = 1 above (two tokens with four loads per batch need 172 VGPRs: two waves per SIMD,
+// 21 us instead of 12 us on an 8B-shaped layer launch).  Cells that are not instantiated stay
+// null.
+constexpr int max_batch_index(int mt) { return mt <= 1 ? 2 : (mt <= 4 ? 1 : 0); }
 
 template <int BITS, int MT>
 void fill_table_row(KernelTable<BITS> &t) {
@@ -508,8 +510,6 @@ Geometry pick_geometry(int M, int N, int K, int lds_limit, const Tuning &tu) {
     const bool pair_odd = BITS == 2 && g.mt == 1 && it >= 3;
     g.batch_index = (it % 4 == 0 || it >= 8) ? 2 : ((it % 2 == 0 || pair_odd) ? 1 : 0);
     if (g.batch_index > max_batch_index(g.mt)) g.batch_index = max_batch_index(g.mt);
-    // (1-bit chunks unpack to twice the registers: four loads per batch spill from two tokens on)
-    if (BITS == 1 && g.mt >= 2 && g.batch_index > 1) g.batch_index = 1;
     const int rpw = 64 >> g.lpr_log2;
     const long wave_passes = ((long)N + rpw - 1) / rpw;
 
