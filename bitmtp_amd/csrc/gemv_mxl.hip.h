@@ -13,9 +13,10 @@
 //   * weights, scales and activations are read through buffer resources: rows past N and
 //     tokens past M read as zero by the range check, so there are no clamps or selects in the
 //     address arithmetic, and a load is one per-lane offset plus a scalar;
-//   * one workgroup per 16 rows and no striding loop (four waves per SIMD: at five the
-//     registers that hold a tile's activations between load and staging spill, which puts a
-//     memory round trip in front of every tile and costs 40 % at eight tokens);
+//   * one workgroup per 16 rows and no striding loop, and a register budget that lets every
+//     workgroup of a layer-sized launch be resident at once (template parameters NB and OCC
+//     below; a build that spills the staged-activation registers puts a memory round trip in
+//     front of every tile and costs 40 % at eight tokens);
 //   * after the K-slice exchange wave r finishes result column r of every token quad, so the
 //     epilogue (division, rounding, store) is spread over the four waves.
 // Same summation order as gemv_mx.hip.h; the final division by the activation multiplier is an
