@@ -425,7 +425,7 @@ def main() -> int:
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "traffic": None if traffic is None else round(traffic),
         "kernel": (f"gemv_dot4_grouped_kernel<BITS=2, MT={dom}>" if dom <= 2
-                   else "gemv_mxl_kernel<BITS=2, MR=4, W=4>") + f" (grouped, 7 descriptors, width {dom})",
+                   else "gemv_mxl_kernel<BITS=2, MR=4, SF16=false, W=4, NB=1, OCC=5>") + f" (grouped, 7 descriptors, width {dom})",
         "bytes_per_launch": bytes_per_launch,
         "us_per_launch": per_width[dom]["us_per_launch"],
         "read_probe_us": per_width[dom]["read_probe_us"],
