@@ -165,11 +165,13 @@ def test_t2_decode_widths_merged_shapes(oracle, M, N, K):
 @pytest.mark.parametrize("bits,M,N,K", [(2, 3, 12288, 4096), (2, 16, 9728, 9728), (2, 17, 12288, 4096),
                                          (2, 8, 24576, 4096), (2, 2, 2048, 6144), (2, 2, 2560, 9728),
                                          (1, 2, 9728, 9728), (1, 16, 12288, 4096), (2, 32, 19456, 2560),
-                                         (2, 33, 4100, 5120)])
+                                         (2, 33, 4100, 5120),
+                                         (2, 9, 19456, 2560), (2, 9, 24576, 4096), (1, 9, 19456, 2560)])
 def test_larger_single_matrices_and_two_token_long_rows(oracle, bits, M, N, K):
     """Single matrices with more 16-row tiles than CUs and long rows (several K tiles per wave of
     the lean matrix-core kernel, two and three token tiles), the two-token blocks that go to the
-    matrix cores for K >= 4096, and the 32-row prefill width on the widest merged matrix."""
+    matrix cores for K >= 4096, the 32-row prefill width on the widest merged matrix, and nine tokens
+    on matrices with more than four row tiles per CU (the 96-register build of the lean kernel)."""
     p = oracle.synth_problem(300 + M + N // 7, M, N, K, bits)
     check_problem(oracle, p, bits, "large-single")
 
