@@ -35,3 +35,32 @@ def test_cli_needs_exactly_one_of_preset_and_shapes(monkeypatch, capsys):
     assert gb.main() == 2
     monkeypatch.setattr("sys.argv", ["gemv_bench", "--preset", "head", "--shapes", "128x128"])
     assert gb.main() == 2
+
+
+def test_bench_refuses_more_than_one_gpu(capsys):
+    """bench.py is a one-GPU measurement: any other --gpus exits with a message and status 2
+    before anything touches a device."""
+    import subprocess
+    import sys
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode == 2 and "one GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_traffic_table_matches_the_layer_bytes():
+    """The measured HBM traffic bench.py reports comes from profiles/traffic.json; every width's
+    figure is the counters' own arithmetic and lies within 10 % above the algorithmic bytes."""
+    import bench
+    for width in (1, 4, 8):
+        t = bench.measured_traffic(width)
+        assert t is not None and bench.LAYER_BYTES <= t <= 1.10 * bench.LAYER_BYTES
+    assert bench.measured_traffic(5) is None
+    assert bench.LAYER_BYTES == sum(bench.t2_bytes(n, k) for _, n, k in bench.PROJECTIONS) == 13369344
+
+
+def test_kernel_choices_of_the_sweep_tool():
+    from bitmtp_amd import gemv_bench
+    assert gemv_bench.KERNELS["auto"] == (0, 0)
+    assert set(gemv_bench.KERNELS) >= {"auto", "dot4", "staged", "operand", "lean", "stream", "single-token"}
