@@ -10,10 +10,17 @@
 //                                   ws bf16 [N, K/128]) -> bf16 [.., N]
 //   bonsai::q1g128_int8xint1_linear(a_int8 [.., K], b_packed int8 [N, K/8], s, ws) -> bf16 [.., N]
 //   bonsai::quant_input(x [.., K]) -> (q int8 [.., K], s f32 [.., 1])      (model.py:632-636)
+//   bonsai::fused_norm_quant(x bf16 [.., K], w bf16 [K], eps) -> (q, s)                 (model.py:307-319)
+//   bonsai::fused_add_norm_quant(x, residual, w, eps) -> (h bf16 [.., K], q, s)          (model.py:322-336)
+//   bonsai::silu_mul_quant(gate_up bf16 [.., 2F]) -> (q int8 [.., F], s f32 [.., 1])     (model.py:1058-1061)
 #include <ATen/ATen.h>
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
+
+#include <initializer_list>
+#include <tuple>
+#include <vector>
 
 #include "../../include/bonsai_gemv.h"
 
@@ -104,22 +111,117 @@ std::tuple<at::Tensor, at::Tensor> quant_input_cuda(const at::Tensor &x) {
 
 std::tuple<at::Tensor, at::Tensor> quant_input_meta(const at::Tensor &x) { return quant_shapes(x); }
 
+// ---- fused producers ---------------------------------------------------------------------
+void check_bf16_rows(const char *op, const at::Tensor &x, const at::Tensor &w) {
+    TORCH_CHECK(x.dim() >= 1 && x.scalar_type() == at::kBFloat16, op, ": expected a bf16 tensor of rank >= 1");
+    const int64_t k = x.size(-1);
+    TORCH_CHECK(k >= 8 && k % 8 == 0, op, ": the last dimension must be a multiple of 8");
+    TORCH_CHECK(w.scalar_type() == at::kBFloat16 && w.dim() == 1 && w.size(0) == k, op, ": weight must be bf16 [K]");
+}
+
+std::vector<int64_t> with_last(const at::Tensor &x, int64_t last) {
+    std::vector<int64_t> shape(x.sizes().begin(), x.sizes().end());
+    shape.back() = last;
+    return shape;
+}
+
+void check_cuda_contiguous(const char *op, std::initializer_list<const at::Tensor *> ts) {
+    const at::Tensor *first = *ts.begin();
+    for (const at::Tensor *t : ts)
+        TORCH_CHECK(t->is_cuda() && t->is_contiguous() && t->device() == first->device(), op,
+                    ": expected contiguous CUDA tensors on one device");
+}
+
+std::tuple<at::Tensor, at::Tensor> norm_quant_meta(const at::Tensor &x, const at::Tensor &w, double) {
+    check_bf16_rows("fused_norm_quant", x, w);
+    return {at::empty(x.sizes(), x.options().dtype(at::kChar)),
+            at::empty(with_last(x, 1), x.options().dtype(at::kFloat))};
+}
+
+std::tuple<at::Tensor, at::Tensor> norm_quant_cuda(const at::Tensor &x, const at::Tensor &w, double eps) {
+    auto [q, s] = norm_quant_meta(x, w, eps);
+    check_cuda_contiguous("fused_norm_quant", {&x, &w});
+    const int64_t k = x.size(-1), m = x.numel() / k;
+    if (m == 0) return {q, s};
+    c10::DeviceGuard guard(x.device());
+    const int rc = bonsai_rmsnorm_quant_int8(x.data_ptr(), w.data_ptr(), (float)eps, static_cast<int8_t *>(q.data_ptr()),
+                                             static_cast<float *>(s.data_ptr()), (int)m, (int)k,
+                                             c10::hip::getCurrentHIPStream().stream());
+    TORCH_CHECK(rc == 0, "fused_norm_quant: native launch failed with status ", rc);
+    return {q, s};
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor> add_norm_quant_meta(const at::Tensor &x, const at::Tensor &residual,
+                                                                   const at::Tensor &w, double) {
+    check_bf16_rows("fused_add_norm_quant", x, w);
+    TORCH_CHECK(residual.scalar_type() == at::kBFloat16 && residual.sizes() == x.sizes(),
+                "fused_add_norm_quant: residual must match x");
+    return {at::empty(x.sizes(), x.options()), at::empty(x.sizes(), x.options().dtype(at::kChar)),
+            at::empty(with_last(x, 1), x.options().dtype(at::kFloat))};
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor> add_norm_quant_cuda(const at::Tensor &x, const at::Tensor &residual,
+                                                                   const at::Tensor &w, double eps) {
+    auto [h, q, s] = add_norm_quant_meta(x, residual, w, eps);
+    check_cuda_contiguous("fused_add_norm_quant", {&x, &residual, &w});
+    const int64_t k = x.size(-1), m = x.numel() / k;
+    if (m == 0) return {h, q, s};
+    c10::DeviceGuard guard(x.device());
+    const int rc = bonsai_add_rmsnorm_quant_int8(x.data_ptr(), residual.data_ptr(), w.data_ptr(), (float)eps,
+                                                 h.data_ptr(), static_cast<int8_t *>(q.data_ptr()),
+                                                 static_cast<float *>(s.data_ptr()), (int)m, (int)k,
+                                                 c10::hip::getCurrentHIPStream().stream());
+    TORCH_CHECK(rc == 0, "fused_add_norm_quant: native launch failed with status ", rc);
+    return {h, q, s};
+}
+
+std::tuple<at::Tensor, at::Tensor> silu_mul_quant_meta(const at::Tensor &gate_up) {
+    TORCH_CHECK(gate_up.dim() >= 1 && gate_up.scalar_type() == at::kBFloat16,
+                "silu_mul_quant: expected a bf16 tensor of rank >= 1");
+    const int64_t f2 = gate_up.size(-1);
+    TORCH_CHECK(f2 >= 16 && f2 % 16 == 0, "silu_mul_quant: last dimension must be 2F with F a multiple of 8");
+    return {at::empty(with_last(gate_up, f2 / 2), gate_up.options().dtype(at::kChar)),
+            at::empty(with_last(gate_up, 1), gate_up.options().dtype(at::kFloat))};
+}
+
+std::tuple<at::Tensor, at::Tensor> silu_mul_quant_cuda(const at::Tensor &gate_up) {
+    auto [q, s] = silu_mul_quant_meta(gate_up);
+    check_cuda_contiguous("silu_mul_quant", {&gate_up});
+    const int64_t f2 = gate_up.size(-1), m = gate_up.numel() / f2;
+    if (m == 0) return {q, s};
+    c10::DeviceGuard guard(gate_up.device());
+    const int rc = bonsai_silu_mul_quant_int8(gate_up.data_ptr(), static_cast<int8_t *>(q.data_ptr()),
+                                              static_cast<float *>(s.data_ptr()), (int)m, (int)(f2 / 2),
+                                              c10::hip::getCurrentHIPStream().stream());
+    TORCH_CHECK(rc == 0, "silu_mul_quant: native launch failed with status ", rc);
+    return {q, s};
+}
+
 }  // namespace
 
 TORCH_LIBRARY(bonsai, m) {
     m.def("t2g128_int8xint2_linear(Tensor a_int8, Tensor b_packed, Tensor s, Tensor ws) -> Tensor");
     m.def("q1g128_int8xint1_linear(Tensor a_int8, Tensor b_packed, Tensor s, Tensor ws) -> Tensor");
     m.def("quant_input(Tensor x) -> (Tensor, Tensor)");
+    m.def("fused_norm_quant(Tensor x, Tensor w, float eps) -> (Tensor, Tensor)");
+    m.def("fused_add_norm_quant(Tensor x, Tensor residual, Tensor w, float eps) -> (Tensor, Tensor, Tensor)");
+    m.def("silu_mul_quant(Tensor gate_up) -> (Tensor, Tensor)");
 }
 
 TORCH_LIBRARY_IMPL(bonsai, CUDA, m) {
     m.impl("t2g128_int8xint2_linear", &gemv_cuda<2>);
     m.impl("q1g128_int8xint1_linear", &gemv_cuda<1>);
     m.impl("quant_input", &quant_input_cuda);
+    m.impl("fused_norm_quant", &norm_quant_cuda);
+    m.impl("fused_add_norm_quant", &add_norm_quant_cuda);
+    m.impl("silu_mul_quant", &silu_mul_quant_cuda);
 }
 
 TORCH_LIBRARY_IMPL(bonsai, Meta, m) {
     m.impl("t2g128_int8xint2_linear", &gemv_meta<2>);
     m.impl("q1g128_int8xint1_linear", &gemv_meta<1>);
     m.impl("quant_input", &quant_input_meta);
+    m.impl("fused_norm_quant", &norm_quant_meta);
+    m.impl("fused_add_norm_quant", &add_norm_quant_meta);
+    m.impl("silu_mul_quant", &silu_mul_quant_meta);
 }

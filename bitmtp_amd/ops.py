@@ -154,7 +154,8 @@ def torch_ops_lib_path() -> str:
 
 def load_torch_ops():
     """Registers the dispatcher operators ``torch.ops.bonsai.t2g128_int8xint2_linear``,
-    ``q1g128_int8xint1_linear`` and ``quant_input`` (CUDA and Meta kernels; csrc/torch_ops.cpp)
+    ``q1g128_int8xint1_linear``, ``quant_input``, ``fused_norm_quant``, ``fused_add_norm_quant``
+    and ``silu_mul_quant`` (CUDA and Meta kernels; csrc/torch_ops.cpp)
     and returns the ``torch.ops.bonsai`` namespace.  Same tensors in and out as the functions of
     this module (reference: model.py:118-268,632-636); a missing library raises."""
     global _torch_ops_loaded

@@ -28,6 +28,11 @@ def test_schemas(bonsai):
     assert str(bonsai.q1g128_int8xint1_linear.default._schema) == \
         "bonsai::q1g128_int8xint1_linear(Tensor a_int8, Tensor b_packed, Tensor s, Tensor ws) -> Tensor"
     assert str(bonsai.quant_input.default._schema) == "bonsai::quant_input(Tensor x) -> (Tensor, Tensor)"
+    assert str(bonsai.fused_norm_quant.default._schema) == \
+        "bonsai::fused_norm_quant(Tensor x, Tensor w, float eps) -> (Tensor, Tensor)"
+    assert str(bonsai.fused_add_norm_quant.default._schema) == \
+        "bonsai::fused_add_norm_quant(Tensor x, Tensor residual, Tensor w, float eps) -> (Tensor, Tensor, Tensor)"
+    assert str(bonsai.silu_mul_quant.default._schema) == "bonsai::silu_mul_quant(Tensor gate_up) -> (Tensor, Tensor)"
 
 
 @pytest.mark.parametrize("bits", [1, 2])
@@ -66,6 +71,28 @@ def test_quant_input_meta(bonsai):
         assert s.shape == (2, 7, 1) and s.dtype == torch.float32
     with pytest.raises(RuntimeError, match="bf16, fp16 or fp32"):
         bonsai.quant_input(torch.empty(2, 128, dtype=torch.int32, device="meta"))
+
+
+def test_fused_producers_meta(bonsai):
+    """Shapes and dtypes of the fused producers as the reference's helpers return them
+    (model.py:307-336, 1058-1061), and their argument checks."""
+    x = torch.empty(2, 3, 2048, dtype=torch.bfloat16, device="meta")
+    w = torch.empty(2048, dtype=torch.bfloat16, device="meta")
+    q, s = bonsai.fused_norm_quant(x, w, 1e-6)
+    assert q.shape == x.shape and q.dtype == torch.int8 and s.shape == (2, 3, 1) and s.dtype == torch.float32
+    h, q, s = bonsai.fused_add_norm_quant(x, x, w, 1e-6)
+    assert h.shape == x.shape and h.dtype == torch.bfloat16 and q.dtype == torch.int8 and s.shape == (2, 3, 1)
+    gu = torch.empty(5, 2 * 6144, dtype=torch.bfloat16, device="meta")
+    q, s = bonsai.silu_mul_quant(gu)
+    assert q.shape == (5, 6144) and q.dtype == torch.int8 and s.shape == (5, 1)
+    with pytest.raises(RuntimeError, match="weight must be bf16"):
+        bonsai.fused_norm_quant(x, w[:1024], 1e-6)
+    with pytest.raises(RuntimeError, match="residual must match"):
+        bonsai.fused_add_norm_quant(x, x[:1], w, 1e-6)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        bonsai.silu_mul_quant(torch.empty(5, 24, dtype=torch.bfloat16, device="meta"))
+    with pytest.raises(RuntimeError, match="bf16"):
+        bonsai.silu_mul_quant(torch.empty(5, 32, dtype=torch.float32, device="meta"))
 
 
 def test_cpu_tensors_have_no_kernel(bonsai):
@@ -121,3 +148,22 @@ def test_registered_ops_under_graph_capture(bonsai):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y.view(torch.int16), eager.view(torch.int16)), rep
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M, K", [(1, 2048), (9, 2560), (4, 6144)])
+def test_registered_producers_equal_the_ctypes_operators(bonsai, M, K):
+    g = torch.Generator(device="cpu").manual_seed(M * 7 + K)
+    x = torch.randn(M, K, generator=g).to("cuda", torch.bfloat16)
+    r = torch.randn(M, K, generator=g).to("cuda", torch.bfloat16)
+    w = (torch.rand(K, generator=g) + 0.5).to("cuda", torch.bfloat16)
+    q0, s0 = ops.fused_norm_quant(x, w, 1e-6)
+    q1, s1 = bonsai.fused_norm_quant(x, w, 1e-6)
+    assert torch.equal(q0, q1) and torch.equal(s0, s1)
+    h0, q0, s0 = ops.fused_add_norm_quant(x, r, w, 1e-6)
+    h1, q1, s1 = bonsai.fused_add_norm_quant(x, r, w, 1e-6)
+    assert torch.equal(h0.view(torch.int16), h1.view(torch.int16)) and torch.equal(q0, q1) and torch.equal(s0, s1)
+    gu = torch.randn(M, 2 * K, generator=g).to("cuda", torch.bfloat16)
+    q0, s0 = ops.silu_mul_quant(gu)
+    q1, s1 = bonsai.silu_mul_quant(gu)
+    assert q1.shape == (M, K) and torch.equal(q0, q1) and torch.equal(s0, s1)
