@@ -237,3 +237,22 @@ def test_narrow_grouped_fp16_scales_and_graph_replay(oracle):
         torch.cuda.synchronize()
         for a, b in zip(outs, eager):
             assert torch.equal(a, b), f"replay {rep} differs"
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+@pytest.mark.parametrize("seed", [11, 12, 13, 14])
+def test_random_descriptor_sets(oracle, bits, seed):
+    """Seeded random calls: 1 to 20 descriptors with any mix of widths 1..17, ragged row counts
+    and K from 128 to 6144 -- narrow and wide blocks in one call, token tiling, more descriptors
+    than one launch of either grouped kernel holds, shapes that fall back to the single-GEMV
+    path -- each descriptor checked against the oracle as a GEMV of its own."""
+    rng = np.random.default_rng(seed * 10 + bits)
+    count = int(rng.integers(1, 21))
+    ks = [128, 384, 512, 1024, 1536, 2048, 2560, 4096, 6144]
+    probs = []
+    for i in range(count):
+        m = int(rng.choice([1, 1, 2, 3, 4, 8, 9, 16, 17]))
+        n = int(rng.integers(1, 700))
+        k = int(rng.choice(ks))
+        probs.append(oracle.synth_problem(seed * 1000 + i, m, n, k, bits))
+    check_group(oracle, probs, bits, f"random set seed={seed}")
