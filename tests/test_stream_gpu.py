@@ -205,3 +205,51 @@ def test_read_probe_runs_and_writes_nothing(nbytes, workgroups, persistent):
     assert rc == 0
     torch.cuda.synchronize()
     assert int(sink.item()) == 0 and torch.equal(buf, before)
+
+
+def test_first_launch_on_a_capturing_stream_is_refused():
+    """In a fresh process whose first GEMV launch arrives while the stream is being captured,
+    the entry points return status 3 and enqueue nothing (the one-time set-up changes kernel
+    attributes, which must not happen under capture); after `t2g128_init` outside capture the
+    same call is captured and replays with the eager result."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = r'''
+import ctypes, sys, torch
+sys.path.insert(0, %r)
+from bitmtp_amd import ops
+lib = ops.t2_lib()
+M, N, K = 4, 256, 2048
+g0 = torch.Generator().manual_seed(1)
+a = torch.randint(-128, 128, (M, K), generator=g0, dtype=torch.int8).cuda()
+b = torch.randint(-128, 128, (N, K // 4), generator=g0, dtype=torch.int8).cuda()
+s = torch.full((M, 1), 3.0, dtype=torch.float32).cuda()
+ws = torch.full((N, K // 128), 0.02, dtype=torch.bfloat16).cuda()
+out = torch.zeros(M, N, dtype=torch.bfloat16).cuda()
+def call():
+    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return lib.t2g128_gemv_ex(a.data_ptr(), b.data_ptr(), out.data_ptr(), s.data_ptr(), ws.data_ptr(),
+                              M, N, K, 0, 0, sp)
+torch.cuda.synchronize()
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph):
+    rc_captured = call()
+assert rc_captured == 3, rc_captured
+graph.replay(); torch.cuda.synchronize()
+assert not out.any()                      # nothing was enqueued
+assert lib.t2g128_init() == 0
+assert call() == 0
+torch.cuda.synchronize()
+eager = out.clone(); out.zero_()
+graph2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph2):
+    assert call() == 0
+graph2.replay(); torch.cuda.synchronize()
+assert eager.any() and torch.equal(out.view(torch.int16), eager.view(torch.int16))
+print("REFUSED-THEN-OK")
+''' % root
+    proc = subprocess.run([sys.executable, "-c", script], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                          text=True, timeout=110)
+    assert proc.returncode == 0 and "REFUSED-THEN-OK" in proc.stdout, proc.stderr[-1500:]
