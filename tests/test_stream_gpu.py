@@ -253,3 +253,48 @@ print("REFUSED-THEN-OK")
     proc = subprocess.run([sys.executable, "-c", script], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
                           text=True, timeout=110)
     assert proc.returncode == 0 and "REFUSED-THEN-OK" in proc.stdout, proc.stderr[-1500:]
+
+
+def test_first_launches_from_two_threads():
+    """Two host threads make the library's first launches at the same moment (ctypes releases
+    the interpreter lock during the call): the one-time set-up runs under a lock, both calls
+    succeed and both results equal a later single-threaded call."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = r'''
+import ctypes, sys, threading, torch
+sys.path.insert(0, %r)
+from bitmtp_amd import ops
+lib = ops.t2_lib()
+M, N, K = 9, 512, 2048
+g0 = torch.Generator().manual_seed(2)
+a = torch.randint(-128, 128, (M, K), generator=g0, dtype=torch.int8).cuda()
+b = torch.randint(-128, 128, (N, K // 4), generator=g0, dtype=torch.int8).cuda()
+s = torch.full((M, 1), 5.0, dtype=torch.float32).cuda()
+ws = torch.full((N, K // 128), 0.03, dtype=torch.bfloat16).cuda()
+outs = [torch.zeros(M, N, dtype=torch.bfloat16).cuda() for _ in range(3)]
+streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+torch.cuda.synchronize()
+rcs = [None, None]
+barrier = threading.Barrier(2)
+def work(i):
+    barrier.wait()
+    rcs[i] = lib.t2g128_gemv_ex(a.data_ptr(), b.data_ptr(), outs[i].data_ptr(), s.data_ptr(), ws.data_ptr(),
+                                M, N, K, 0, 0, ctypes.c_void_p(streams[i].cuda_stream))
+ts = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+[t.start() for t in ts]; [t.join() for t in ts]
+torch.cuda.synchronize()
+assert rcs == [0, 0], rcs
+sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+assert lib.t2g128_gemv_ex(a.data_ptr(), b.data_ptr(), outs[2].data_ptr(), s.data_ptr(), ws.data_ptr(), M, N, K, 0, 0, sp) == 0
+torch.cuda.synchronize()
+assert outs[2].any()
+assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+assert torch.equal(outs[1].view(torch.int16), outs[2].view(torch.int16))
+print("TWO-THREADS-OK")
+''' % root
+    proc = subprocess.run([sys.executable, "-c", script], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                          text=True, timeout=110)
+    assert proc.returncode == 0 and "TWO-THREADS-OK" in proc.stdout, proc.stderr[-1500:]
