@@ -23,6 +23,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "../../include/bonsai_decode.h"
 #include "wave_reduce.h"
 
@@ -1087,7 +1090,8 @@ bf16_linear_kernel(const uint16_t *x, const uint16_t *w, uint16_t *out, int M, i
 }
 
 constexpr int kMaxDevices = 16;
-bool g_lin_ready[kMaxDevices];
+std::atomic<bool> g_lin_ready[kMaxDevices];  // set last, under g_lin_mutex
+std::mutex g_lin_mutex;
 int g_lin_cus[kMaxDevices];
 int g_lin_lds[kMaxDevices];
 
@@ -1245,7 +1249,7 @@ fp8_linear_kernel(const uint8_t *x, const float *x_scale, const uint8_t *w, floa
     }
 }
 
-bool g_fp8_ready[kMaxDevices];
+std::atomic<bool> g_fp8_ready[kMaxDevices];  // set last, under g_lin_mutex
 
 int g_rows_per_wave = 0;  // 0 = heuristic; set through bonsai_decode_set_tuning
 int g_attn_engine = 0;    // 0 = matrix-core chunk pass, 1 = VALU chunk pass
@@ -1443,7 +1447,7 @@ extern "C" int bonsai_draft_chain_ws(const void *logits, int rows, int ld, int v
 // ---------------------------------------------------------------------------
 constexpr int kStaticScratchFloats = BONSAI_MAX_WIDTH * kDraftSplits * 4;  // 16 KiB
 static __device__ __align__(256) float scratch[kStaticScratchFloats];
-static float *g_static_scratch[kMaxDevices];  // device address of `scratch`, per device
+std::atomic<float *> g_static_scratch[kMaxDevices];  // the array's address on each device (every thread resolves the same value)
 
 extern "C" int bonsai_draft_chain_static(const void *logits, int rows, int ld, int vocab,
                                          float threshold, int32_t *tokens, float *conf,
@@ -1455,14 +1459,14 @@ extern "C" int bonsai_draft_chain_static(const void *logits, int rows, int ld, i
     if ((size_t)rows * kDraftSplits * 4 > (size_t)kStaticScratchFloats) return BONSAI_DECODE_ERR_ARG;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
-    if (g_static_scratch[dev] == nullptr) {
+    if (g_static_scratch[dev].load(std::memory_order_acquire) == nullptr) {
         float *ptr = nullptr;
         if (hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess ||
             ptr == nullptr)
             return BONSAI_DECODE_ERR_LAUNCH;
-        g_static_scratch[dev] = ptr;
+        g_static_scratch[dev].store(ptr, std::memory_order_release);
     }
-    float *ws = g_static_scratch[dev];
+    float *ws = g_static_scratch[dev].load(std::memory_order_acquire);
     hipStream_t st = static_cast<hipStream_t>(stream);
     // every slot the merge reads is written by the split pass of the same call: nothing to clear
     hipLaunchKernelGGL(draft_rows_split_kernel, dim3(rows * kDraftSplits), dim3(kDraftSplitThreads), 0,
@@ -1480,7 +1484,8 @@ extern "C" int bonsai_bf16_linear(const void *x, const void *w, void *out, int M
     if (M < 1 || M > BONSAI_MAX_WIDTH || N < 1 || K < 64 || K % 64 != 0) return BONSAI_DECODE_ERR_ARG;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
-    if (!g_lin_ready[dev]) {
+    if (!g_lin_ready[dev].load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_lin_mutex);  // one-time set-up: call once before capturing
         int cus = 0, lds = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
             hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
@@ -1490,7 +1495,7 @@ extern "C" int bonsai_bf16_linear(const void *x, const void *w, void *out, int M
             return BONSAI_DECODE_ERR_LAUNCH;
         g_lin_cus[dev] = cus > 0 ? cus : 1;
         g_lin_lds[dev] = lds;
-        g_lin_ready[dev] = true;
+        g_lin_ready[dev].store(true, std::memory_order_release);
     }
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return BONSAI_DECODE_ERR_ARG;
     const int nwaves = K % 512 == 0 ? 8 : (K % 256 == 0 ? 4 : (K % 128 == 0 ? 2 : 1));
@@ -1537,7 +1542,8 @@ extern "C" int bonsai_fp8_linear(const void *x, const float *x_scale, const void
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return BONSAI_DECODE_ERR_ARG;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
-    if (!g_fp8_ready[dev]) {
+    if (!g_fp8_ready[dev].load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_lin_mutex);
         int cus = 0, lds = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
             hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
@@ -1547,7 +1553,7 @@ extern "C" int bonsai_fp8_linear(const void *x, const float *x_scale, const void
             return BONSAI_DECODE_ERR_LAUNCH;
         g_lin_cus[dev] = cus > 0 ? cus : 1;
         g_lin_lds[dev] = lds;
-        g_fp8_ready[dev] = true;
+        g_fp8_ready[dev].store(true, std::memory_order_release);
     }
     const int nwaves = K % 1024 == 0 ? 8 : (K % 512 == 0 ? 4 : (K % 256 == 0 ? 2 : 1));
     const int ntiles = (N + 15) / 16;
