@@ -183,28 +183,12 @@ class Runner:
 
 
 def read_probe_us(torch, ops_mod, run, nbytes: int, workgroups: int, persistent: bool, dev) -> float:
-    """Microseconds per launch of the library's read probe (bonsai_read_probe: the same bytes
+    """Microseconds per launch of the read probe of the bench-only probe library (the same bytes
     read once from HBM with the GEMV's launch shape and no arithmetic), timed like every other
     figure here: one graph of launches over >= 512 MB of distinct buffers, best of 5 replays."""
-    probe = ops_mod.t2_lib().bonsai_read_probe
-    n = max(2, -(-MIN_DISTINCT_BYTES // nbytes))
-    bufs = torch.empty(n, nbytes, dtype=torch.uint8, device=dev).random_(0, 256)
-    sink = torch.zeros(1, dtype=torch.int32, device=dev)
-    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    rc = probe(bufs[0].data_ptr(), nbytes, workgroups, int(persistent), sink.data_ptr(), sp)
-    if rc != 0:
-        raise RuntimeError(f"bonsai_read_probe returned {rc}")
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        spc = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        for i in range(n):
-            probe(bufs[i].data_ptr(), nbytes, workgroups, int(persistent), sink.data_ptr(), spc)
-    g.replay()
-    torch.cuda.synchronize()
-    t, _ = run.time_stats(g)
-    del g, bufs
-    return t / n * 1e6
+    from bitmtp_amd import probe
+    return probe.read_probe_us(torch, nbytes, workgroups, persistent, dev, MIN_DISTINCT_BYTES)
+
 
 def cpu_baseline(budget_s: float):
     """Times the C oracle (OpenMP over output rows) on one layer at widths 1, 4, 8 --

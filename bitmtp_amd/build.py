@@ -20,12 +20,14 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 
-# source (under csrc/) -> library (under the package)
+# source (under csrc/, or a path relative to the package) -> library (under the package)
 TARGETS = {
     "t2g128_kernels.hip": os.path.join("t2g128_kernels", "libbonsai_t2.so"),
     "q1g128_kernels.hip": os.path.join("q1g128_kernels", "libbonsai_q1.so"),
     "act_quant.hip": os.path.join("act_quant", "libbonsai_actq.so"),
     "decode_ops.hip": os.path.join("decode_ops", "libbonsai_decode.so"),
+    # measurement aids of the benchmarks, apart from the drop-in libraries
+    os.path.join("..", "bench_probe", "bench_probe.hip"): os.path.join("bench_probe", "libbonsai_probe.so"),
 }
 
 HIPCC_FLAGS = [
@@ -45,9 +47,10 @@ def lib_path(source: str) -> str:
 
 
 def _deps() -> list[str]:
+    probe = os.path.join(HERE, "bench_probe")
     return [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [
-        os.path.join(HERE, "..", "include", "bonsai_gemv.h"),
-        os.path.join(HERE, "..", "include", "bonsai_decode.h")]
+        os.path.join(probe, f) for f in os.listdir(probe) if f.endswith((".hip", ".h"))] + [
+        os.path.join(HERE, "..", "include", h) for h in ("bonsai_gemv.h", "bonsai_decode.h", "bonsai_probe.h")]
 
 
 def _stale(out: str) -> bool:

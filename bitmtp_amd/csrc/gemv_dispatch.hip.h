@@ -44,25 +44,26 @@ using Dot4GroupFn = void (*)(int, int, int, int, int, int, int, int, int, int, i
 
 template <int BITS>
 struct Dot4GroupKernels {
-    Dot4GroupFn fn[kDot4GroupMaxWidth][kBatchKinds][2];  // [MT - 1][U index][scale kind]
+    Dot4GroupFn fn[kDot4GroupMaxWidth][kBatchKinds][kVariants];  // [MT - 1][U index][bf16 / fp16 scales / group sums]
 };
+
+template <int BITS, int MT, int U, int UI>
+void fill_dot4_group_cell(Dot4GroupKernels<BITS> &x) {
+    x.fn[MT - 1][UI][0] = gemv_dot4_grouped_kernel<BITS, MT, U, false, false>;
+    x.fn[MT - 1][UI][1] = gemv_dot4_grouped_kernel<BITS, MT, U, true, false>;
+    x.fn[MT - 1][UI][2] = gemv_dot4_grouped_kernel<BITS, MT, U, false, true>;
+}
 
 template <int BITS>
 const Dot4GroupKernels<BITS> &dot4_group_kernels() {
     static const Dot4GroupKernels<BITS> t = [] {
         Dot4GroupKernels<BITS> x{};
-        x.fn[0][0][0] = gemv_dot4_grouped_kernel<BITS, 1, 1, false>;
-        x.fn[0][0][1] = gemv_dot4_grouped_kernel<BITS, 1, 1, true>;
-        x.fn[0][1][0] = gemv_dot4_grouped_kernel<BITS, 1, 2, false>;
-        x.fn[0][1][1] = gemv_dot4_grouped_kernel<BITS, 1, 2, true>;
-        x.fn[0][2][0] = gemv_dot4_grouped_kernel<BITS, 1, 4, false>;
-        x.fn[0][2][1] = gemv_dot4_grouped_kernel<BITS, 1, 4, true>;
-        x.fn[1][0][0] = gemv_dot4_grouped_kernel<BITS, 2, 1, false>;
-        x.fn[1][0][1] = gemv_dot4_grouped_kernel<BITS, 2, 1, true>;
-        x.fn[1][1][0] = gemv_dot4_grouped_kernel<BITS, 2, 2, false>;
-        x.fn[1][1][1] = gemv_dot4_grouped_kernel<BITS, 2, 2, true>;
-        x.fn[1][2][0] = gemv_dot4_grouped_kernel<BITS, 2, 2, false>;  // (never picked: two tokens take
-        x.fn[1][2][1] = gemv_dot4_grouped_kernel<BITS, 2, 2, true>;   //  at most two loads per batch)
+        fill_dot4_group_cell<BITS, 1, 1, 0>(x);
+        fill_dot4_group_cell<BITS, 1, 2, 1>(x);
+        fill_dot4_group_cell<BITS, 1, 4, 2>(x);
+        fill_dot4_group_cell<BITS, 2, 1, 0>(x);
+        fill_dot4_group_cell<BITS, 2, 2, 1>(x);
+        fill_dot4_group_cell<BITS, 2, 2, 2>(x);  // (never picked: two tokens take at most two loads per batch)
         return x;
     }();
     return t;
@@ -73,7 +74,7 @@ int dot4_group_init_device(int max_lds) {
     const Dot4GroupKernels<BITS> &t = dot4_group_kernels<BITS>();
     for (int mt = 0; mt < kDot4GroupMaxWidth; ++mt)
         for (int u = 0; u < kBatchKinds; ++u)
-            for (int sk = 0; sk < 2; ++sk)
+            for (int sk = 0; sk < kVariants; ++sk)
                 if (hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[mt][u][sk]),
                                         hipFuncAttributeMaxDynamicSharedMemorySize,
                                         max_lds) != hipSuccess)
@@ -89,7 +90,7 @@ int dot4_group_init_device(int max_lds) {
 template <int BITS>
 int launch_dot4_grouped(const GemvProblem *probs, int count, int out_kind, int scale_kind,
                         int lds_limit, hipStream_t stream) {
-    if (count < 1 || count > kDot4GroupMax || out_kind == OUT_G32) return -1;
+    if (count < 1 || count > kDot4GroupMax) return -1;
     int mt = 1;
     for (int i = 0; i < count; ++i) mt = probs[i].M > mt ? probs[i].M : mt;
     if (mt > kDot4GroupMaxWidth) return -1;
@@ -151,10 +152,12 @@ int launch_dot4_grouped(const GemvProblem *probs, int count, int out_kind, int s
         ends[i] = wg;
     }
     for (int i = count; i < kDot4GroupMax; ++i) ends[i] = 0x7fffffff;
-    const Dot4GroupFn fn = dot4_group_kernels<BITS>().fn[mt - 1][batch_index][scale_kind];
+    const Dot4GroupFn fn = dot4_group_kernels<BITS>().fn[mt - 1][batch_index][out_kind == OUT_G32 ? 2 : scale_kind];
     hipLaunchKernelGGL(fn, dim3(wg, 1, 1), dim3(waves * 64, 1, 1), lds, stream, ends[0], ends[1],
                        ends[2], ends[3], ends[4], ends[5], ends[6], ends[7], ends[8], ends[9],
                        ends[10], ends[11], out_kind == OUT_F32 ? 1 : 0, waves * 64, tbl);
+    note_kernel("gemv_dot4_grouped_kernel", BITS, mt, batch_index == 2 && mt == 1 ? 4 : (batch_index >= 1 ? 2 : 1),
+                scale_kind == 1 && out_kind != OUT_G32, out_kind == OUT_G32);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
@@ -307,6 +310,9 @@ int launch_matrix_core(int engine, bool single_tile, const int8_t *A, const uint
     hipLaunchKernelGGL(fn, dim3(grid_x, ntok_tiles, 1), dim3(nw * 64, 1, 1), lds_for(ri, mt),
                        stream, args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
                        args.mt, args.ks_log2, args.out_f32, args.passes, args.div_magic);
+    note_kernel(flex ? "gemv_mfma_direct_flex_kernel" : (direct ? (nw == 8 ? "gemv_mfma_direct8_kernel" : "gemv_mfma_direct_kernel")
+                                                                : "gemv_mfma_kernel"),
+                BITS, 1 << ri, variant == 1, variant == 2);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
@@ -334,7 +340,7 @@ int launch_grouped_mx_only(const GemvProblem &q, int out_kind, int scale_kind, i
     }
     // the lean form where it applies (every token tile of at most 16, a layer-sized matrix)
     const MxTuning &gtu = mx_tuning<BITS>();
-    if (out_kind != OUT_G32 && nb <= kMxlMaxDesc && gtu.row_tiles == 0 && gtu.max_wgs == 0) {
+    if (nb <= kMxlMaxDesc && gtu.row_tiles == 0 && gtu.max_wgs == 0) {
         bool ok = true;
         for (int i = 0; i < nb; ++i) ok = ok && mxl_problem_ok<BITS>(batch[i]);
         if (ok) {
@@ -393,7 +399,7 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
     // form of the same kernel already ran).
     const long lean_tiles = (long)((M + kMfmaTokens - 1) / kMfmaTokens) * ((N + 15) / 16);
     const bool lean_default = mtu.engine == 0 && M >= min_width && N <= kLongMatrixRows &&
-                              out_kind != OUT_G32 && lean_tiles <= 8L * st.n_cus[dev];
+                              lean_tiles <= 8L * st.n_cus[dev];
     if ((mtu.engine == 4 || lean_default) && M >= min_width) {
         // the grouped kernel with a single descriptor
         const GemvProblem q{A, B, out, s, ws, M, N, K};
@@ -423,7 +429,8 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
 // Problems the grouped kernel takes (K % 512 == 0, aligned operands) share launches of up to
 // kMxMaxDesc descriptors each, blocks wider than 16 tokens as several token tiles; the rest
 // go through launch_gemv one by one.  The arithmetic of every problem is that of the
-// single-GEMV entry points.
+// single-GEMV entry points: identical int32 group sums; the fp32 value has the same bits where
+// the same kernel and geometry serve both, and differs by summation order only elsewhere.
 template <int BITS>
 int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_kind,
                    hipStream_t stream) {
@@ -462,6 +469,12 @@ int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_
         }
         if (rc == -1)
             rc = launch_mx<BITS>(batch, nb, out_kind, scale_kind, lds_limit, st.n_cus[dev], stream);
+        if (rc == -1) {  // no grouped kernel takes the batch: its problems one by one
+            rc = 0;
+            for (int i = 0; i < nb && rc == 0; ++i)
+                rc = launch_gemv<BITS>(batch[i].A, batch[i].B, batch[i].out, batch[i].s, batch[i].ws,
+                                       batch[i].M, batch[i].N, batch[i].K, out_kind, scale_kind, stream);
+        }
         nb = 0;
         return rc;
     };
@@ -469,7 +482,7 @@ int launch_grouped(const GemvProblem *probs, int count, int out_kind, int scale_
     // (a forced smallest width of the matrix-core kernel, tu.min_width > 0, keeps them there)
     GemvProblem nbatch[kDot4GroupMax];
     int nnb = 0;
-    const bool narrow_on = out_kind != OUT_G32 && tu.min_width <= 0;
+    const bool narrow_on = tu.min_width <= 0;
     auto flush_n = [&]() -> int {
         if (nnb == 0) return 0;
         int rc = launch_dot4_grouped<BITS>(nbatch, nnb, out_kind, scale_kind, lds_limit, stream);

@@ -519,6 +519,7 @@ int launch_mx(const GemvProblem *probs, int count, int out_kind, int scale_kind,
     const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
     const MxKernelFn fn = mx_table<BITS>().fn[ri][variant];
     hipLaunchKernelGGL(fn, dim3(wg, 1, 1), dim3(kMxThreads, 1, 1), lds, stream, prm);
+    note_kernel("gemv_mx_kernel", BITS, R, variant == 1, variant == 2);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

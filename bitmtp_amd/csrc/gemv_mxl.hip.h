@@ -74,7 +74,9 @@ __host__ __device__ constexpr size_t mxl_lds_bytes(int mmax, int waves) {
 // at exactly 96 registers, which costs about 0.1 us on launches that have no fifth workgroup per
 // CU to place, and saves a microsecond on those that do (19456 x 2560 at nine tokens 8.6 ->
 // 7.6 us), so the host picks per launch.
-template <int BITS, int MR, bool SF16, int W, int NB, int OCC>
+// G32: store the exact int32 group sums G[m][n][g] (what the matrix cores return, before any
+// scale) instead of the scaled result; the scales and multipliers are not read.
+template <int BITS, int MR, bool SF16, int W, int NB, int OCC, bool G32 = false>
 __global__ void __launch_bounds__(W * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, int e8, int e9,
                 int e10, int e11, int out_f32, int mmax, const MxlTable tbl) {
@@ -110,8 +112,9 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
         const_cast<int8_t *>(d.A), 0, M * K, kMxlBufferWord3);
     const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t *>(d.B), 0, N * row_bytes, kMxlBufferWord3);
+    // (no records when the group sums are wanted: every scale reads as zero, no access is made)
     const __amdgpu_buffer_rsrc_t rS = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(d.ws), 0, N * G * 2, kMxlBufferWord3);
+        const_cast<uint16_t *>(d.ws), 0, G32 ? 0 : N * G * 2, kMxlBufferWord3);
 
     // ---- weight tile: kLoads coalesced 16-byte loads per lane, one 8-byte scale load
     uint32_t w_off[MF::kLoads];
@@ -172,7 +175,7 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
     if (NB > 1 && nbatch > 1) act_load(amore, tb, 1);
     load_w(tb);
     float s_tok = 1.0f;
-    if (wave < MR) {
+    if (!G32 && wave < MR) {
         const int tkc = 4 * kb + wave;
         s_tok = d.s[tkc < M ? tkc : M - 1];
     }
@@ -226,12 +229,23 @@ gemv_mxl_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, 
             const v4i vb1 = {(int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
             v4i dd = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, vb0, vcr, 0, 0, 0);
             dd = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, vb1, dd, 0, 0, 0);
+            if (G32) {
+                const int row = n0 + op_row;
+#pragma unroll
+                for (int r = 0; r < MR; ++r) {
+                    const int tk = 4 * kb + r;
+                    if (row < N && tk < M)
+                        reinterpret_cast<int32_t *>(d.out)[((size_t)tk * N + row) * G + (kt * kMxTileGroups + gi)] = dd[r];
+                }
+                continue;
+            }
             const uint32_t raw = (gi & 2) ? sc.y : sc.x;
             const float wsf = scale_to_f32<SF16>((uint16_t)((gi & 1) ? (raw >> 16) : (raw & 0xffffu)));
 #pragma unroll
             for (int r = 0; r < MR; ++r) acc[r] += (float)dd[r] * wsf;
         }
     }
+    if (G32) return;
 
     // ---- K slices added in slice order; wave r finishes column r of every token quad
 #pragma unroll
@@ -266,6 +280,11 @@ constexpr int kMxlWideWaves = 12;
 // dense: more than four workgroups per CU to place (only matters for width class 2)
 template <int BITS, int W, int OCC1, int OCC2>
 MxlKernelFn mxl_kernel_w(int scale_kind, int width_class) {
+    if (scale_kind == 2) {  // int32 group sums from the same builds
+        if (width_class == 0) return gemv_mxl_kernel<BITS, 1, false, W, 1, OCC1, true>;
+        if (width_class == 1) return gemv_mxl_kernel<BITS, 4, false, W, 1, OCC1, true>;
+        return gemv_mxl_kernel<BITS, 4, false, W, 2, OCC2, true>;
+    }
     if (width_class == 0)
         return scale_kind == 1 ? gemv_mxl_kernel<BITS, 1, true, W, 1, OCC1> : gemv_mxl_kernel<BITS, 1, false, W, 1, OCC1>;
     if (width_class == 1)
@@ -281,7 +300,7 @@ MxlKernelFn mxl_kernel(int scale_kind, int width_class, bool wide, bool dense) {
 
 template <int BITS>
 int mxl_init_device(int max_lds) {
-    for (int sk = 0; sk < 2; ++sk)
+    for (int sk = 0; sk < 3; ++sk)
         for (int wc = 0; wc < 3; ++wc)
             for (int wide = 0; wide < 2; ++wide)
                 for (int dense = 0; dense < 2; ++dense)
@@ -293,7 +312,7 @@ int mxl_init_device(int max_lds) {
 }
 
 // True when this kernel takes the problem: what gemv_mx.hip.h takes, with at most 16 tokens and
-// operand sizes within the 32-bit buffer range.
+// operand sizes within the 32-bit buffer range (q.ws may be null when group sums are wanted).
 template <int BITS>
 bool mxl_problem_ok(const GemvProblem &q) {
     return mx_problem_ok(q, false) && q.M <= 16 && (long)q.N * (q.K * BITS / 8) < (1L << 31) &&
@@ -305,7 +324,7 @@ bool mxl_problem_ok(const GemvProblem &q) {
 template <int BITS>
 int launch_mxl(const GemvProblem *probs, int count, int out_kind, int scale_kind, int lds_limit,
                int n_cus, hipStream_t stream) {
-    if (count < 1 || count > kMxlMaxDesc || out_kind == OUT_G32) return -1;
+    if (count < 1 || count > kMxlMaxDesc) return -1;
     long wgs = 0;
     int mmax = 1;
     bool one_token = true;
@@ -354,10 +373,15 @@ int launch_mxl(const GemvProblem *probs, int count, int out_kind, int scale_kind
         ends[i] = wg;
     }
     for (int i = count; i < kMxlMaxDesc; ++i) ends[i] = 0x7fffffff;
-    hipLaunchKernelGGL(mxl_kernel<BITS>(scale_kind, one_token ? 0 : (mmax <= 8 ? 1 : 2), wide, dense), dim3(wg, 1, 1), dim3(waves * 64, 1, 1),
+    const int width_class = one_token ? 0 : (mmax <= 8 ? 1 : 2);
+    const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
+    hipLaunchKernelGGL(mxl_kernel<BITS>(variant, width_class, wide, dense), dim3(wg, 1, 1), dim3(waves * 64, 1, 1),
                        lds, stream, ends[0], ends[1], ends[2], ends[3], ends[4], ends[5], ends[6],
                        ends[7], ends[8], ends[9], ends[10], ends[11], out_kind == OUT_F32 ? 1 : 0,
                        mmax, tbl);
+    // <BITS, MR, SF16, W, NB, OCC, G32> as instantiated by mxl_kernel
+    note_kernel("gemv_mxl_kernel", BITS, width_class == 0 ? 1 : 4, scale_kind == 1 && variant != 2, waves,
+                width_class == 2 ? 2 : 1, wide ? 3 : (width_class == 2 && !dense ? 4 : 5), variant == 2);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

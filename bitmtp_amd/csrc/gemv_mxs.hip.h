@@ -45,7 +45,9 @@ __host__ __device__ constexpr size_t mxs_lds_bytes(int M, int K) {
 // MR: result columns kept per lane.  A lane's MFMA result holds tokens 4 (lane / 16) + r,
 // r = 0..3; a single-token block needs only r = 0 (MR = 1), which saves three of the four
 // convert / multiply-add pairs per group.
-template <int BITS, bool SF16, int MR>
+// G32: store the exact int32 group sums G[m][n][g] instead of the scaled result (scales and
+// multipliers are not read).
+template <int BITS, bool SF16, int MR, bool G32 = false>
 __global__ void __launch_bounds__(kMxThreads) __attribute__((amdgpu_waves_per_eu(4)))
 gemv_mxs_kernel(const MxsParams p) {
     using MF = MfmaFmt<BITS>;
@@ -109,7 +111,7 @@ gemv_mxs_kernel(const MxsParams p) {
 #pragma unroll
         for (int h = 0; h < MF::kLoads; ++h)
             tr.w[h] = *reinterpret_cast<const u32x4 *>(bw + (last ? voff_w_last[h] : voff_w[h]));
-        tr.sc = *reinterpret_cast<const uint2 *>(bs + (last ? voff_sc_last : voff_sc));
+        if (!G32) tr.sc = *reinterpret_cast<const uint2 *>(bs + (last ? voff_sc_last : voff_sc));
     };
     auto park_tile = [&](const TileRegs &tr) {
 #pragma unroll
@@ -162,7 +164,7 @@ gemv_mxs_kernel(const MxsParams p) {
 #pragma unroll
     for (int r = 0; r < MR; ++r) {
         const int m = 4 * kb + r;
-        rinv[r] = p.s[m < M ? m : M - 1];
+        rinv[r] = G32 ? 1.0f : p.s[m < M ? m : M - 1];
     }
     __builtin_amdgcn_sched_barrier(0);
     TileRegs ring[kMxsRing];
@@ -227,7 +229,7 @@ gemv_mxs_kernel(const MxsParams p) {
             // (the copy is pinned to its own registers here: otherwise the compiler lets the
             // reload below land in temporaries and moves them at the end of the trip, behind a
             // wait for every load in flight)
-            uint2 sc = ring[j].sc;
+            uint2 sc = G32 ? make_uint2(0u, 0u) : ring[j].sc;
             asm volatile("" : "+v"(sc.x), "+v"(sc.y));
             load_tile(ring[j], l_rt, l_kt);
             advance_load();
@@ -255,6 +257,16 @@ gemv_mxs_kernel(const MxsParams p) {
                 const v4i vb1 = {(int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
                 v4i dd = __builtin_amdgcn_mfma_i32_16x16x64_i8(va0, vb0, vcr, 0, 0, 0);
                 dd = __builtin_amdgcn_mfma_i32_16x16x64_i8(va1, vb1, dd, 0, 0, 0);
+                if (G32) {
+                    const int row = (c_rt << 4) + op_row;
+#pragma unroll
+                    for (int r = 0; r < MR; ++r) {
+                        const int tk = 4 * kb + r;
+                        if (row < N && tk < M)
+                            reinterpret_cast<int32_t *>(p.out)[((size_t)tk * N + row) * G + (c_kt * kMxTileGroups + gi)] = dd[r];
+                    }
+                    continue;
+                }
                 const uint32_t raw = (gi & 2) ? sc.y : sc.x;
                 const float wsf =
                     scale_to_f32<SF16>((uint16_t)((gi & 1) ? (raw >> 16) : (raw & 0xffffu)));
@@ -263,7 +275,7 @@ gemv_mxs_kernel(const MxsParams p) {
             }
             if (++c_kt == KT) {  // uniform: the row tile is complete
                 const int row = (c_rt << 4) + op_row;
-                const bool row_ok = row < N;
+                const bool row_ok = row < N && !G32;
 #pragma unroll
                 for (int r = 0; r < MR; ++r) {
                     const int tk = 4 * kb + r;
@@ -291,6 +303,8 @@ using MxsKernelFn = void (*)(const MxsParams);
 
 template <int BITS>
 MxsKernelFn mxs_kernel(int scale_kind, bool one_token) {
+    if (scale_kind == 2)  // int32 group sums
+        return one_token ? gemv_mxs_kernel<BITS, false, 1, true> : gemv_mxs_kernel<BITS, false, 4, true>;
     if (one_token)
         return scale_kind == 1 ? gemv_mxs_kernel<BITS, true, 1> : gemv_mxs_kernel<BITS, false, 1>;
     return scale_kind == 1 ? gemv_mxs_kernel<BITS, true, 4> : gemv_mxs_kernel<BITS, false, 4>;
@@ -298,7 +312,7 @@ MxsKernelFn mxs_kernel(int scale_kind, bool one_token) {
 
 template <int BITS>
 int mxs_init_device(int max_lds) {
-    for (int sk = 0; sk < 2; ++sk)
+    for (int sk = 0; sk < 3; ++sk)
         for (int one = 0; one < 2; ++one)
             if (hipFuncSetAttribute(reinterpret_cast<const void *>(mxs_kernel<BITS>(sk, one != 0)),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -334,7 +348,10 @@ int mxs_wgs_per_cu(const GemvProblem &q, int lds_limit) {
 // `forced`) a matrix long enough that every resident wave gets at least two row tiles.
 template <int BITS>
 bool mxs_problem_ok(const GemvProblem &q, int out_kind, int lds_limit, int n_cus, bool forced) {
-    if (out_kind == OUT_G32 || q.M > 16 || !mx_problem_ok(q, false)) return false;
+    (void)out_kind;  // every output kind, the int32 group sums included
+    if (q.M > 16 || !mx_problem_ok(q, false)) return false;
+    // tile offsets are 32-bit: the packed matrix and its scale table stay below 4 GiB
+    if ((long)q.N * (q.K * BITS / 8) >= (1L << 32) || (long)q.N * (q.K / kGroup) * 2 >= (1L << 32)) return false;
     if (mxs_wgs_per_cu<BITS>(q, lds_limit) < 2) return false;
     if (forced) return true;
     const MxsTuning &tu = mxs_tuning<BITS>();
@@ -361,8 +378,10 @@ int launch_mxs(const GemvProblem &q, int out_kind, int scale_kind, int lds_limit
     const int n_rt = (q.N + 15) / 16;
     int wgs = n_cus * mxs_wgs_per_cu<BITS>(q, lds_limit);
     if (wgs * kMxWaves > n_rt) wgs = (n_rt + kMxWaves - 1) / kMxWaves;
-    hipLaunchKernelGGL(mxs_kernel<BITS>(scale_kind, q.M == 1), dim3(wgs, 1, 1), dim3(kMxThreads, 1, 1),
+    const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
+    hipLaunchKernelGGL(mxs_kernel<BITS>(variant, q.M == 1), dim3(wgs, 1, 1), dim3(kMxThreads, 1, 1),
                        mxs_lds_bytes<BITS>(q.M, q.K), stream, prm);
+    note_kernel("gemv_mxs_kernel", BITS, variant == 1, q.M == 1 ? 1 : 4, variant == 2);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

@@ -62,7 +62,8 @@ __device__ __forceinline__ u32x4 nibble_planes16(const u32x4 in) {
     return r;
 }
 
-template <int LPR_LOG2, bool SF16>
+// G32: store the exact int32 group sums G[0][n][g] instead of the scaled result.
+template <int LPR_LOG2, bool SF16, bool G32 = false>
 __global__ void __launch_bounds__(kRowregThreads) __attribute__((amdgpu_waves_per_eu(4)))
 gemv_rowreg_kernel(const RowregParams p) {
     constexpr int LPR = 1 << LPR_LOG2;   // lanes per row = scale groups per row
@@ -83,7 +84,7 @@ gemv_rowreg_kernel(const RowregParams p) {
     const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t *>(p.B), 0, N * row_bytes, kRowregBufferWord3);
     const __amdgpu_buffer_rsrc_t rS = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(p.ws), 0, N * G * 2, kRowregBufferWord3);
+        const_cast<uint16_t *>(p.ws), 0, G32 ? 0 : N * G * 2, kRowregBufferWord3);
 
     struct Batch {
         u32x4 w[kRowregU][2];
@@ -117,7 +118,7 @@ gemv_rowreg_kernel(const RowregParams p) {
         planes[tid] = nibble_planes16(in);
         qsum[tid] = sum4_i8(in.x) + sum4_i8(in.y) + sum4_i8(in.z) + sum4_i8(in.w);
     }
-    const float rinv = __builtin_amdgcn_rcpf(p.s[0]);
+    const float rinv = G32 ? 1.0f : __builtin_amdgcn_rcpf(p.s[0]);
     __syncthreads();
     uint32_t act[2][16];
     int asum = 0;
@@ -151,12 +152,18 @@ gemv_rowreg_kernel(const RowregParams p) {
                 }
             }
             const int g = (ah << 4) + (int)al;  // the exact group sum
+            if (G32) {
+                const int row = bb * BR + u * RPW + lr;
+                if (row < N) reinterpret_cast<int32_t *>(p.out)[(size_t)row * G + lc] = g;
+                res[u] = 0.0f;
+                continue;
+            }
             res[u] = row_lanes_sum((float)g * scale_to_f32<SF16>(t.sc[u]), LPR_LOG2);
         }
 #pragma unroll
         for (int u = 0; u < kRowregU; ++u) {
             const int row = bb * BR + u * RPW + lr;
-            if (lc == 0 && row < N) {
+            if (!G32 && lc == 0 && row < N) {
                 const float yv = res[u] * rinv;
                 if (p.out_f32)
                     reinterpret_cast<float *>(p.out)[row] = yv;
@@ -185,6 +192,14 @@ using RowregKernelFn = void (*)(const RowregParams);
 
 inline RowregKernelFn rowreg_kernel(int K, int scale_kind) {
     const bool f16 = scale_kind == 1;
+    if (scale_kind == 2) {  // int32 group sums
+        switch (K) {
+        case 1024: return gemv_rowreg_kernel<3, false, true>;
+        case 2048: return gemv_rowreg_kernel<4, false, true>;
+        case 4096: return gemv_rowreg_kernel<5, false, true>;
+        default: return nullptr;
+        }
+    }
     switch (K) {
     case 1024: return f16 ? gemv_rowreg_kernel<3, true> : gemv_rowreg_kernel<3, false>;
     case 2048: return f16 ? gemv_rowreg_kernel<4, true> : gemv_rowreg_kernel<4, false>;
@@ -200,7 +215,8 @@ inline bool rowreg_problem_ok(const GemvProblem &q, int out_kind, bool forced) {
     const auto al = [](const void *ptr, uintptr_t a) {
         return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) == 0;
     };
-    if (out_kind == OUT_G32 || q.M != 1 || rowreg_kernel(q.K, 0) == nullptr) return false;
+    (void)out_kind;  // every output kind, the int32 group sums included
+    if (q.M != 1 || rowreg_kernel(q.K, 0) == nullptr) return false;
     if (!al(q.A, 16) || !al(q.B, 16) || !al(q.ws, 2)) return false;
     if ((long)q.N * (q.K / 4) >= (1L << 31)) return false;
     return forced || (long)q.N * (q.K / 4) >= (32L << 20);
@@ -223,8 +239,10 @@ inline int launch_rowreg(const GemvProblem &q, int out_kind, int scale_kind, int
     int wgs = n_cus * (wgs_per_cu > 0 ? wgs_per_cu : 4);
     const int need = (n_batch + 3) / 4;
     if (wgs > need) wgs = need;
-    hipLaunchKernelGGL(rowreg_kernel(q.K, scale_kind), dim3(wgs, 1, 1), dim3(kRowregThreads, 1, 1), 0,
+    const int variant = out_kind == OUT_G32 ? 2 : scale_kind;
+    hipLaunchKernelGGL(rowreg_kernel(q.K, variant), dim3(wgs, 1, 1), dim3(kRowregThreads, 1, 1), 0,
                        stream, prm);
+    note_kernel("gemv_rowreg_kernel", 2, lpr == 8 ? 3 : (lpr == 16 ? 4 : 5), variant == 1, variant == 2);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

@@ -39,6 +39,43 @@ constexpr int kMaxThreads = 512;  // workgroup size limit of the kernels
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_G32 = 2 };
 
+// Which kernel the calling thread's last launch went to: the family and its template
+// arguments, kept as numbers and formatted on request.  Tests and benchmarks read it to
+// state (and assert) which kernel a shape reached; nothing in a launch depends on it.
+struct LastKernel {
+    const char *family = "none";
+    int bits = 0;
+    int t[6] = {0, 0, 0, 0, 0, 0};  // template arguments after BITS, -1 = unused
+    int launches = 0;               // launches recorded by this thread so far
+};
+inline LastKernel &last_kernel() {
+    static thread_local LastKernel k;
+    return k;
+}
+inline void note_kernel(const char *family, int bits, int t0 = -1, int t1 = -1, int t2 = -1,
+                        int t3 = -1, int t4 = -1, int t5 = -1) {
+    LastKernel &k = last_kernel();
+    k.family = family;
+    k.bits = bits;
+    k.t[0] = t0;
+    k.t[1] = t1;
+    k.t[2] = t2;
+    k.t[3] = t3;
+    k.t[4] = t4;
+    k.t[5] = t5;
+    ++k.launches;
+}
+// "family<bits,t0,...>" into a thread-local buffer
+inline const char *last_kernel_name() {
+    static thread_local char buf[128];
+    const LastKernel &k = last_kernel();
+    int n = snprintf(buf, sizeof buf, "%s<%d", k.family, k.bits);
+    for (int i = 0; i < 6 && k.t[i] >= 0 && n < (int)sizeof buf; ++i)
+        n += snprintf(buf + n, sizeof buf - n, ",%d", k.t[i]);
+    if (n < (int)sizeof buf) snprintf(buf + n, sizeof buf - n, ">");
+    return buf;
+}
+
 struct GemvArgs {
     const int8_t *A;
     const uint8_t *B;
@@ -322,7 +359,7 @@ struct Dot4GroupTable {
     Dot4GroupDesc d[kDot4GroupMax];
 };
 
-template <int BITS, int MT, int U, bool SF16>
+template <int BITS, int MT, int U, bool SF16, bool G32 = false>
 __global__ void __launch_bounds__(kMaxThreads)
 gemv_dot4_grouped_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6, int e7, int e8,
                          int e9, int e10, int e11, int pout_f32, int pthreads,
@@ -336,7 +373,7 @@ gemv_dot4_grouped_kernel(int e0, int e1, int e2, int e3, int e4, int e5, int e6,
     const Dot4GroupDesc d = tbl.d[di];
     const GemvArgs a{d.A, d.B, d.out, d.s, d.ws, d.M, d.N, d.K, d.lpr_log2_passes & 0xff,
                      d.lpr_log2_passes >> 8, pout_f32, d.div_magic};
-    gemv_dot4_body<BITS, MT, U, false, SF16>(a, wg - d.wg_begin, 0, pthreads, smem);
+    gemv_dot4_body<BITS, MT, U, G32, SF16>(a, wg - d.wg_begin, 0, pthreads, smem);
 }
 
 // ---------------------------------------------------------------------------
@@ -556,6 +593,7 @@ int launch_gemv_dot4(const int8_t *A, const uint8_t *B, void *out, const float *
     hipLaunchKernelGGL(fn, dim3(g.grid_x, g.ntiles, 1), dim3(g.waves * 64, 1, 1), g.lds, stream,
                        args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
                        args.lpr_log2, args.passes, args.out_f32, args.div_magic, g.waves * 64);
+    note_kernel("gemv_dot4_kernel", BITS, g.mt, 1 << g.batch_index, scale_kind == 1 && out_kind != OUT_G32, out_kind == OUT_G32);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

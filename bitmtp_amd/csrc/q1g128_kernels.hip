@@ -80,6 +80,10 @@ void q1g128_w1a16_linear(const void *A, const int8_t *B, void *C, const void *ws
 
 int q1g128_init(void) { return init_all_kernels<1>(); }
 
+const char *q1g128_last_kernel(void) { return last_kernel_name(); }
+
+int q1g128_launch_count(void) { return last_kernel().launches; }
+
 void q1g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes) {
     Tuning &t = lib_state<1>().tuning;
     t.lanes_per_row = lanes_per_row;

@@ -2,7 +2,6 @@
 // gfx950.  Entry points are declared in include/bonsai_gemv.h; the drop-in one
 // replaces src/bonsai_sft/gpu/t2g128_kernels/t2g128_kernels.cu:123-148.
 #include "gemv_dispatch.hip.h"
-#include "read_probe.hip.h"
 
 #include "../../include/bonsai_gemv.h"
 
@@ -11,6 +10,10 @@ using namespace bonsai;
 extern "C" {
 
 int t2g128_init(void) { return init_all_kernels<2>(); }
+
+const char *t2g128_last_kernel(void) { return last_kernel_name(); }
+
+int t2g128_launch_count(void) { return last_kernel().launches; }
 
 void t2g128_set_tuning(int lanes_per_row, int waves_per_wg, int passes) {
     Tuning &t = lib_state<2>().tuning;
@@ -43,11 +46,6 @@ void t2g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width) {
     t.row_tiles = row_tiles;
     t.max_wgs = max_wgs;
     t.min_width = min_width;
-}
-
-int bonsai_read_probe(const void *src, size_t bytes, int workgroups, int persistent, void *sink,
-                      void *stream) {
-    return launch_read_probe(src, bytes, workgroups, persistent, sink, static_cast<hipStream_t>(stream));
 }
 
 void t2g128_set_stream_tuning(int min_bytes, int wgs_per_cu) {

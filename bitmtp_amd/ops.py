@@ -91,9 +91,10 @@ def load_t2_kernel() -> None:
     lib.t2g128_set_grouped_tuning.restype = None
     lib.t2g128_set_stream_tuning.argtypes = [ctypes.c_int] * 2
     lib.t2g128_set_stream_tuning.restype = None
-    lib.bonsai_read_probe.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
-                                      ctypes.c_void_p, ctypes.c_void_p]
-    lib.bonsai_read_probe.restype = ctypes.c_int
+    lib.t2g128_last_kernel.argtypes = []
+    lib.t2g128_last_kernel.restype = ctypes.c_char_p
+    lib.t2g128_launch_count.argtypes = []
+    lib.t2g128_launch_count.restype = ctypes.c_int
     _t2_lib = lib
 
 
@@ -122,6 +123,10 @@ def load_q1_kernel() -> None:
     lib.q1g128_set_grouped_tuning.restype = None
     lib.q1g128_set_stream_tuning.argtypes = [ctypes.c_int] * 2
     lib.q1g128_set_stream_tuning.restype = None
+    lib.q1g128_last_kernel.argtypes = []
+    lib.q1g128_last_kernel.restype = ctypes.c_char_p
+    lib.q1g128_launch_count.argtypes = []
+    lib.q1g128_launch_count.restype = ctypes.c_int
     _q1_lib = lib
 
 
@@ -188,6 +193,20 @@ def actq_lib() -> ctypes.CDLL:
     return _actq_lib
 
 
+def last_kernel(bits: int) -> str:
+    """``family<template arguments>`` of the kernel this thread's last launch through the T2
+    (``bits=2``) or Q1 (``bits=1``) library went to (diagnostics for tests and benchmarks)."""
+    lib = t2_lib() if bits == 2 else q1_lib()
+    fn = lib.t2g128_last_kernel if bits == 2 else lib.q1g128_last_kernel
+    return fn().decode()
+
+
+def launch_count(bits: int) -> int:
+    """Kernel launches this thread has made through the T2 / Q1 library so far."""
+    lib = t2_lib() if bits == 2 else q1_lib()
+    return int((lib.t2g128_launch_count if bits == 2 else lib.q1g128_launch_count)())
+
+
 def init_kernels() -> None:
     """One-time per-device set-up of both GEMV libraries; call before graph capture."""
     if t2_lib().t2g128_init() != 0 or q1_lib().q1g128_init() != 0:
@@ -216,6 +235,25 @@ def _validate_packed_inputs(a, b, s, ws, *, kind, bits, activation_dtype,
         raise RuntimeError(f"{kind}: inputs and scales must be contiguous CUDA tensors")
     if not all(t.device == a.device for t in tensors):
         raise RuntimeError(f"{kind}: inputs and scales must share one CUDA device")
+
+
+def _validate_group_sum_inputs(a, b, *, kind, bits, device=None):
+    """Checks for a call that returns the int32 group sums (no scales are read): the operand
+    checks of ``_validate_packed_inputs`` that concern the activations and the packed weights.
+    Raw pointers of these tensors go to the kernel, so width, dtype, device and contiguity are
+    all checked before any native call."""
+    if a.dim() != 2 or b.dim() != 2:
+        raise ValueError(f"{kind}: expected rank-2 activation and rank-2 weight")
+    n, k = b.shape[0], b.shape[1] * (8 // bits)
+    require_kernel_shape(kind, a.shape[0], n, k)
+    if a.shape[-1] != k:
+        raise RuntimeError(f"{kind}: activation width mismatch: {a.shape[-1]} != {k}")
+    if a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise RuntimeError(f"{kind}: invalid activation or packed-weight dtype")
+    if not (a.is_cuda and b.is_cuda and a.is_contiguous() and b.is_contiguous()):
+        raise RuntimeError(f"{kind}: inputs must be contiguous CUDA tensors")
+    if b.device != a.device or (device is not None and a.device != device):
+        raise RuntimeError(f"{kind}: inputs must share one CUDA device")
 
 
 def _out_shape(a: torch.Tensor, n: int, kind: str) -> Tuple[int, Tuple[int, ...]]:
@@ -315,15 +353,7 @@ def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[tor
         raise ValueError("bits must be 1 (Q1) or 2 (T2)")
     kind = "t2g128" if bits == 2 else "q1"
     if out_kind == OUT_G32:
-        if a_int8.dim() != 2 or b_packed.dim() != 2:
-            raise ValueError(f"{kind}: expected rank-2 activation and rank-2 weight")
-        n, k = b_packed.shape[0], b_packed.shape[1] * (8 // bits)
-        require_kernel_shape(kind, a_int8.shape[0], n, k)
-        if a_int8.shape[-1] != k or a_int8.dtype != torch.int8 or b_packed.dtype != torch.int8:
-            raise RuntimeError(f"{kind}: invalid activation or packed-weight tensor")
-        if not (a_int8.is_cuda and b_packed.is_cuda and a_int8.is_contiguous()
-                and b_packed.is_contiguous()):
-            raise RuntimeError(f"{kind}: inputs must be contiguous CUDA tensors")
+        _validate_group_sum_inputs(a_int8, b_packed, kind=kind, bits=bits)
     else:
         if a_int8.dim() != 2:
             raise ValueError(f"{kind}: expected rank-2 activation")
@@ -362,7 +392,9 @@ def packed_gemv_grouped(problems: Sequence[Tuple[torch.Tensor, torch.Tensor, Opt
     """Several independent GEMVs ``(a_int8 [M,K], b_packed, s, ws)`` in one native call
     (``*_gemv_grouped``): one launch walks the row tiles of all of them.  Widths, row counts
     and K may differ between the problems; every result is what ``packed_gemv_ex`` gives for
-    that problem alone.  ``outs`` supplies preallocated outputs (so that a captured graph
+    that problem alone: the same int32 group sums, and the same fp32 / bf16 bits wherever both
+    calls reach the same kernel with the same geometry (otherwise equal within the tolerance
+    of the fp32 summation order).  ``outs`` supplies preallocated outputs (so that a captured graph
     allocates nothing); otherwise fresh tensors are returned."""
     if bits not in (1, 2):
         raise ValueError("bits must be 1 (Q1) or 2 (T2)")
@@ -381,9 +413,7 @@ def packed_gemv_grouped(problems: Sequence[Tuple[torch.Tensor, torch.Tensor, Opt
         if a.dim() != 2:
             raise ValueError(f"{kind}: expected rank-2 activation")
         if out_kind == OUT_G32:
-            if b.dim() != 2:
-                raise ValueError(f"{kind}: expected rank-2 weight")
-            require_kernel_shape(kind, a.shape[0], b.shape[0], b.shape[1] * (8 // bits))
+            _validate_group_sum_inputs(a, b, kind=kind, bits=bits, device=dev)
         else:
             _validate_packed_inputs(a, b, s, ws, kind=kind, bits=bits, activation_dtype=torch.int8,
                                     scale_dtypes=(torch.bfloat16, torch.float16))

@@ -96,8 +96,9 @@ int q1g128_gemv_ex(const int8_t *A, const uint8_t *B, void *out, const float *s,
  * measurement -- can be handed over together: one grid walks the row tiles of all of them.
  * Every descriptor is an independent GEMV with the operands and the result of the
  * single-GEMV entry points above (same arithmetic: exact int32 group sums, fp32 scale
- * accumulation, division by s[m], bf16 RNE); widths, row counts and K may differ between
- * descriptors.  `descs` is HOST memory and is read before the call returns; the pointers
+ * accumulation, division by s[m], bf16 RNE; bit-identical to the single call only where both
+ * reach the same kernel with the same geometry, otherwise equal within the stated tolerance);
+ * widths, row counts and K may differ between descriptors.  `descs` is HOST memory and is read before the call returns; the pointers
  * inside are device pointers.  out_kind / scale_kind apply to all descriptors. */
 typedef struct bonsai_gemv_desc {
     const int8_t *A;   /* int8 [M, K] */
@@ -166,8 +167,12 @@ int bonsai_silu_mul_quant_int8(const void *gate_up, int8_t *q, float *s, int M, 
 /* Overrides of the built-in kernel choice and launch geometry, for measurements and for the
  * tests that force every kernel onto small shapes.  Not part of the drop-in surface: no
  * reference counterpart, process-wide, not thread-safe, and a value of zero always restores
- * the built-in choice for that field.  Results never depend on them (every kernel computes the
- * arithmetic stated at the top of this file); only speed does.
+ * the built-in choice for that field.  Every kernel computes the arithmetic stated at the top
+ * of this file: the int32 group sums are identical whatever is chosen, while the fp32 value
+ * may differ in its last bits between kernels and geometries (the order of the fp32 additions
+ * over the groups follows the lanes that share a row, and the streaming kernels multiply by
+ * an approximate reciprocal of s[m] where the others divide), always within the stated
+ * tolerance; the same kernel and geometry give the same bits.
  *
  * set_tuning: the dot4 kernel -- lanes per weight row (4..64, power of two), waves per
  *   workgroup (1..16), row passes per wave (>= 1).
@@ -194,16 +199,15 @@ void q1g128_set_grouped_tuning(int row_tiles, int max_wgs, int min_width);
 void t2g128_set_stream_tuning(int min_bytes, int wgs_per_cu);
 void q1g128_set_stream_tuning(int min_bytes, int wgs_per_cu);
 
-/* Measurement aid (libbonsai_t2.so; no reference counterpart, no arithmetic): reads `bytes` of
- * device memory at `src` (16-byte aligned) exactly once with `workgroups` workgroups of 256
- * threads and discards them.  persistent = 0: every thread requests its share up front (at most
- * eight 16-byte loads, else BONSAI_ERR_ARG) -- the launch shape of a layer-sized GEMV;
- * persistent = 1: workgroups loop with eight loads per lane in flight -- the shape of the
- * kernels for very long matrices.  `sink` is 4 writable device bytes (practically never
- * written).  bench.py times it beside the GEMV on the same byte counts: what the machine
- * needs for the bytes alone. */
-int bonsai_read_probe(const void *src, size_t bytes, int workgroups, int persistent, void *sink,
-                      void *stream);
+/* Which kernel the calling thread's last launch through this library went to, as
+ * "family<template arguments>" (a pointer into thread-local storage, valid until the thread's
+ * next call of the same function), and how many kernel launches the thread has made through
+ * the library so far.  Read-only diagnostics for tests and benchmarks, which state and assert
+ * the kernel a shape reaches; no reference counterpart. */
+const char *t2g128_last_kernel(void);
+const char *q1g128_last_kernel(void);
+int t2g128_launch_count(void);
+int q1g128_launch_count(void);
 
 #ifdef __cplusplus
 }

@@ -7,7 +7,7 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("bonsai_gemv.h", "bonsai_decode.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("bonsai_gemv.h", "bonsai_decode.h", "bonsai_probe.h")]
 
 
 def declared_functions():
@@ -15,7 +15,7 @@ def declared_functions():
     for header in HEADERS:
         text = open(header).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names.update(re.findall(r"\b(?:int|void|int64_t)\s+([a-z0-9_]+)\s*\(", text))
+        names.update(re.findall(r"\b(?:int|void|int64_t|const char \*)\s*([a-z0-9_]+)\s*\(", text))
     return sorted(names)
 
 
@@ -24,8 +24,9 @@ def libs():
     from bitmtp_amd import build, ops
     build.build_all(verbose=False)  # compiles only what is missing or out of date
     from bitmtp_amd import decode_ops
+    from bitmtp_amd import probe
     paths = [ops.t2_lib_path(), ops.q1_lib_path(), ops.actq_lib_path(),
-             decode_ops.decode_lib_path()]
+             decode_ops.decode_lib_path(), probe.probe_lib_path()]
     assert all(os.path.exists(p) for p in paths)
     return [ctypes.CDLL(p) for p in paths]
 
@@ -65,7 +66,8 @@ def test_python_binding_sets_argtypes():
 
 
 def test_decode_library_exports_and_binding(libs):
-    assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["bonsai_decode.h", "bonsai_gemv.h"]
+    assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["bonsai_decode.h", "bonsai_gemv.h",
+                                                                  "bonsai_probe.h"]
     dec = libs[3]
     for name in ("bonsai_qk_norm_rope_kv_write", "bonsai_decode_attention",
                  "bonsai_decode_attention_scratch_bytes", "bonsai_kv_commit", "bonsai_draft_chain",
@@ -106,7 +108,9 @@ def test_argument_checks_need_no_gpu():
     assert t2.t2g128_gemv_grouped(d, 0, 0, 0, None) == 1
     # the read probe: null or misaligned pointers, and a one-shot launch of more than eight loads
     # per thread (256 threads x 16 bytes x 8 per workgroup)
-    probe = t2.bonsai_read_probe
+    from bitmtp_amd import probe as probe_mod
+    assert not hasattr(t2, "bonsai_read_probe")  # measurement aids live in their own library
+    probe = probe_mod.probe_lib().bonsai_read_probe
     assert probe(None, 4096, 1, 0, VP(0x40000), None) == 1
     assert probe(VP(0x10000), 4096, 1, 0, None, None) == 1
     assert probe(VP(0x10008), 4096, 1, 0, VP(0x40000), None) == 1

@@ -26,9 +26,14 @@ def check_problem(O, p, bits, label):
     A, B, s, ws = to_dev(p)
     print(f"[case] {label} bits={bits} M={A.shape[0]} N={B.shape[0]} K={A.shape[1]}", flush=True)
     G = ops.packed_gemv_ex(A, B, None, None, bits=bits, out_kind=ops.OUT_G32)
+    k_g = ops.last_kernel(bits)
     y32 = ops.packed_gemv_ex(A, B, s, ws, bits=bits, out_kind=ops.OUT_F32)
     y16 = ops.packed_int8_linear(A, B, s, ws)
+    k_16 = ops.last_kernel(bits)
     torch.cuda.synchronize()
+    # the group sums come from the same kernel build that produces the bf16 result (the names
+    # differ in their last template argument, the output kind, only)
+    assert k_g.rsplit(",", 1)[0] == k_16.rsplit(",", 1)[0], f"{label}: G from {k_g}, bf16 from {k_16}"
     G_ref = O.c_group_sums(p["A"], p["B"], bits)
     y32_ref, y16_ref = O.c_gemv(p["A"], p["B"], p["s"], p["ws"], bits)
     assert np.array_equal(G.cpu().numpy(), G_ref), f"{label}: int32 group sums differ"
@@ -73,15 +78,16 @@ def test_random_shapes(oracle, bits):
 def test_arbitrary_bytes_and_extreme_activations(oracle, bits):
     """Every byte value (T2 code 0 -> -2 included) and activations over all of int8."""
     rng = np.random.default_rng(7)
-    M, N, K = 6, 96, 1536
-    p = oracle.synth_problem(7, M, N, K, bits)
-    p["A"] = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
-    p["A"][0, :] = -128
-    p["A"][1, :] = 127
-    p["B"] = rng.integers(0, 256, size=p["B"].shape, dtype=np.uint8)
-    p["B"][0, :] = 0x00
-    p["B"][1, :] = 0xFF
-    check_problem(oracle, p, bits, "extreme")
+    for M, N, K in ((6, 96, 1536), (6, 96, 2048), (2, 300, 2048), (1, 300, 6144)):
+        p = oracle.synth_problem(7, M, N, K, bits)
+        p["A"] = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+        p["A"][0, :] = -128
+        if M > 1:
+            p["A"][1, :] = 127
+        p["B"] = rng.integers(0, 256, size=p["B"].shape, dtype=np.uint8)
+        p["B"][0, :] = 0x00
+        p["B"][1, :] = 0xFF
+        check_problem(oracle, p, bits, "extreme")
 
 
 @pytest.mark.parametrize("bits", [2, 1])

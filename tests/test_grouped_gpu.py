@@ -26,11 +26,18 @@ def check_group(O, probs, bits, label):
     dev = [to_dev(p) for p in probs]
     shapes = [(p["A"].shape[0], p["B"].shape[0], p["A"].shape[1]) for p in probs]
     print(f"[case] grouped {label} bits={bits} (M,N,K)={shapes}", flush=True)
+    n0 = ops.launch_count(bits)
     G = ops.packed_gemv_grouped([(A, B, None, None) for A, B, s, ws in dev], bits=bits,
                                 out_kind=ops.OUT_G32)
+    k_g, n1 = ops.last_kernel(bits), ops.launch_count(bits)
     y32 = ops.packed_gemv_grouped(dev, bits=bits, out_kind=ops.OUT_F32)
+    n2 = ops.launch_count(bits)
     y16 = ops.packed_gemv_grouped(dev, bits=bits, out_kind=ops.OUT_BF16)
+    k_16 = ops.last_kernel(bits)
     torch.cuda.synchronize()
+    # the group sums take the same launches as the results (same kernel builds, same count)
+    assert k_g.rsplit(",", 1)[0] == k_16.rsplit(",", 1)[0], f"{label}: G from {k_g}, bf16 from {k_16}"
+    assert n1 - n0 == n2 - n1, f"{label}: {n1 - n0} launches for G, {n2 - n1} for the fp32 result"
     for i, p in enumerate(probs):
         G_ref = O.c_group_sums(p["A"], p["B"], bits)
         y32_ref, y16_ref = O.c_gemv(p["A"], p["B"], p["s"], p["ws"], bits)
@@ -109,7 +116,7 @@ def test_grouped_geometries(oracle, bits, row_tiles, max_wgs):
 def test_grouped_arbitrary_bytes_and_extreme_activations(oracle, bits):
     rng = np.random.default_rng(9)
     probs = []
-    for i, (M, N, K) in enumerate([(6, 96, 1536), (1, 40, 512)]):
+    for i, (M, N, K) in enumerate([(6, 96, 1536), (1, 40, 512), (5, 96, 2048), (2, 80, 2048), (1, 50, 6144), (9, 33, 2560)]):
         p = oracle.synth_problem(800 + i, M, N, K, bits)
         p["A"] = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
         p["A"][0, :] = -128

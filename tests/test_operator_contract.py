@@ -114,6 +114,41 @@ def test_validation_messages(fn, bits, kind, monkeypatch):
     assert ops._t2_lib is None and ops._q1_lib is None  # nothing native was loaded
 
 
+@pytest.mark.parametrize("bits,kind", [(2, "t2g128"), (1, "q1")])
+def test_group_sum_calls_check_their_operands_before_any_native_call(bits, kind, monkeypatch):
+    """A call for the int32 group sums reads no scales, but its activations and weights are
+    checked like any other call -- single and grouped alike: raw pointers of these tensors go
+    to the kernel, so a wrong width, dtype, device or stride must raise here."""
+    monkeypatch.setattr(ops, "_t2_lib", None)
+    monkeypatch.setattr(ops, "_q1_lib", None)
+    K, N, M = 2048, 32, 3
+    cols = K * bits // 8
+    a, b = meta((M, K), torch.int8), meta((N, cols), torch.int8)
+
+    def single(a_, b_):
+        return ops.packed_gemv_ex(a_, b_, None, None, bits=bits, out_kind=ops.OUT_G32)
+
+    def grouped(a_, b_):
+        return ops.packed_gemv_grouped([(a_, b_, None, None)], bits=bits, out_kind=ops.OUT_G32)
+
+    for call in (single, grouped):
+        with pytest.raises(RuntimeError, match="activation width mismatch"):
+            call(meta((M, K + 128), torch.int8), b)
+        with pytest.raises(RuntimeError, match="invalid activation or packed-weight dtype"):
+            call(meta((M, K), torch.uint8), b)
+        with pytest.raises(RuntimeError, match="invalid activation or packed-weight dtype"):
+            call(a, meta((N, cols), torch.uint8))
+        with pytest.raises(ValueError, match="rank-2"):
+            call(meta((1, M, K), torch.int8), b)
+        with pytest.raises(RuntimeError, match="must be contiguous CUDA tensors"):
+            call(a, b)  # meta tensors are not CUDA tensors
+        with pytest.raises(RuntimeError, match="must be contiguous CUDA tensors"):
+            call(torch.zeros(M, K, dtype=torch.int8), torch.zeros(N, cols, dtype=torch.int8))
+        with pytest.raises(RuntimeError, match="must be contiguous CUDA tensors"):
+            call(torch.zeros(M, 2 * K, dtype=torch.int8)[:, ::2], torch.zeros(N, cols, dtype=torch.int8))
+    assert ops._t2_lib is None and ops._q1_lib is None  # nothing native was loaded
+
+
 def test_dispatcher_by_packed_width():
     a = meta((1, 256), torch.int8)
     with pytest.raises(ValueError, match="unknown packed weight layout"):

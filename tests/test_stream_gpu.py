@@ -196,12 +196,12 @@ def test_read_probe_runs_and_writes_nothing(nbytes, workgroups, persistent):
     """The measurement aid reads its buffer (including a ragged tail) and leaves the sink and the
     buffer as they were."""
     import ctypes
-    from bitmtp_amd import ops
+    from bitmtp_amd import probe
     buf = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
     before = buf.clone()
     sink = torch.zeros(1, dtype=torch.int32, device="cuda")
     sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    rc = ops.t2_lib().bonsai_read_probe(buf.data_ptr(), nbytes, workgroups, persistent, sink.data_ptr(), sp)
+    rc = probe.probe_lib().bonsai_read_probe(buf.data_ptr(), nbytes, workgroups, persistent, sink.data_ptr(), sp)
     assert rc == 0
     torch.cuda.synchronize()
     assert int(sink.item()) == 0 and torch.equal(buf, before)
