@@ -214,7 +214,7 @@ def forced_engine():
 
 @pytest.mark.parametrize("bits", [2, 1])
 @pytest.mark.parametrize("M,N,K", [(1, 3000, 2048), (4, 4099, 2048), (8, 2000, 2560), (9, 1500, 6144),
-                                   (16, 700, 9728), (2, 1030, 2048)])
+                                   (16, 700, 4096), (4, 700, 9728), (2, 1030, 2048)])
 def test_streaming_kernel(oracle, forced_engine, bits, M, N, K):
     import bitmtp_amd as ops
     forced_engine(5)
