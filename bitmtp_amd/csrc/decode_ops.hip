@@ -1449,6 +1449,23 @@ constexpr int kStaticScratchFloats = BONSAI_MAX_WIDTH * kDraftSplits * 4;  // 16
 static __device__ __align__(256) float scratch[kStaticScratchFloats];
 std::atomic<float *> g_static_scratch[kMaxDevices];  // the array's address on each device (every thread resolves the same value)
 
+// Looks the array's device address up for the current device `dev` and keeps it.
+static int resolve_static_scratch(int dev) {
+    float *ptr = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess ||
+        ptr == nullptr)
+        return BONSAI_DECODE_ERR_LAUNCH;
+    g_static_scratch[dev].store(ptr, std::memory_order_release);
+    return BONSAI_DECODE_OK;
+}
+
+extern "C" int bonsai_decode_init(void) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
+    if (g_static_scratch[dev].load(std::memory_order_acquire) != nullptr) return BONSAI_DECODE_OK;
+    return resolve_static_scratch(dev);
+}
+
 extern "C" int bonsai_draft_chain_static(const void *logits, int rows, int ld, int vocab,
                                          float threshold, int32_t *tokens, float *conf,
                                          int32_t *accept, void *stream) {
@@ -1459,15 +1476,17 @@ extern "C" int bonsai_draft_chain_static(const void *logits, int rows, int ld, i
     if ((size_t)rows * kDraftSplits * 4 > (size_t)kStaticScratchFloats) return BONSAI_DECODE_ERR_ARG;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
+    hipStream_t st = static_cast<hipStream_t>(stream);
     if (g_static_scratch[dev].load(std::memory_order_acquire) == nullptr) {
-        float *ptr = nullptr;
-        if (hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess ||
-            ptr == nullptr)
-            return BONSAI_DECODE_ERR_LAUNCH;
-        g_static_scratch[dev].store(ptr, std::memory_order_release);
+        // the one-time address lookup is not made on a capturing stream: call bonsai_decode_init
+        // (or this entry point once) before the capture
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+            return BONSAI_DECODE_ERR_NOT_INIT;
+        const int rc = resolve_static_scratch(dev);
+        if (rc != BONSAI_DECODE_OK) return rc;
     }
     float *ws = g_static_scratch[dev].load(std::memory_order_acquire);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     // every slot the merge reads is written by the split pass of the same call: nothing to clear
     hipLaunchKernelGGL(draft_rows_split_kernel, dim3(rows * kDraftSplits), dim3(kDraftSplitThreads), 0,
                        st, static_cast<const uint16_t *>(logits), ld, vocab, kDraftSplits, ws);
@@ -1478,24 +1497,34 @@ extern "C" int bonsai_draft_chain_static(const void *logits, int rows, int ld, i
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
 }
 
+// One-time set-up shared by the bf16 and the FP8 projection: device properties and the LDS limit
+// of `kernel`, under the lock, with the flag checked again inside it (a second thread that
+// waited for the lock finds the work done) and written last.
+static int lin_setup_once(int dev, std::atomic<bool> &ready, const void *kernel) {
+    if (ready.load(std::memory_order_acquire)) return BONSAI_DECODE_OK;
+    std::lock_guard<std::mutex> lock(g_lin_mutex);
+    if (ready.load(std::memory_order_acquire)) return BONSAI_DECODE_OK;
+    int cus = 0, lds = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+        return BONSAI_DECODE_ERR_LAUNCH;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        return BONSAI_DECODE_ERR_LAUNCH;
+    g_lin_cus[dev] = cus > 0 ? cus : 1;
+    g_lin_lds[dev] = lds;
+    ready.store(true, std::memory_order_release);
+    return BONSAI_DECODE_OK;
+}
+
 extern "C" int bonsai_bf16_linear(const void *x, const void *w, void *out, int M, int N, int K,
                                   void *stream) {
     if (!x || !w || !out) return BONSAI_DECODE_ERR_ARG;
     if (M < 1 || M > BONSAI_MAX_WIDTH || N < 1 || K < 64 || K % 64 != 0) return BONSAI_DECODE_ERR_ARG;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
-    if (!g_lin_ready[dev].load(std::memory_order_acquire)) {
-        std::lock_guard<std::mutex> lock(g_lin_mutex);  // one-time set-up: call once before capturing
-        int cus = 0, lds = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
-            return BONSAI_DECODE_ERR_LAUNCH;
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(bf16_linear_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return BONSAI_DECODE_ERR_LAUNCH;
-        g_lin_cus[dev] = cus > 0 ? cus : 1;
-        g_lin_lds[dev] = lds;
-        g_lin_ready[dev].store(true, std::memory_order_release);
+    {   // one-time set-up: call once before capturing
+        const int rc = lin_setup_once(dev, g_lin_ready[dev], reinterpret_cast<const void *>(bf16_linear_kernel));
+        if (rc != BONSAI_DECODE_OK) return rc;
     }
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return BONSAI_DECODE_ERR_ARG;
     const int nwaves = K % 512 == 0 ? 8 : (K % 256 == 0 ? 4 : (K % 128 == 0 ? 2 : 1));
@@ -1542,18 +1571,9 @@ extern "C" int bonsai_fp8_linear(const void *x, const float *x_scale, const void
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return BONSAI_DECODE_ERR_ARG;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BONSAI_DECODE_ERR_LAUNCH;
-    if (!g_fp8_ready[dev].load(std::memory_order_acquire)) {
-        std::lock_guard<std::mutex> lock(g_lin_mutex);
-        int cus = 0, lds = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
-            return BONSAI_DECODE_ERR_LAUNCH;
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(fp8_linear_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return BONSAI_DECODE_ERR_LAUNCH;
-        g_lin_cus[dev] = cus > 0 ? cus : 1;
-        g_lin_lds[dev] = lds;
-        g_fp8_ready[dev].store(true, std::memory_order_release);
+    {
+        const int rc = lin_setup_once(dev, g_fp8_ready[dev], reinterpret_cast<const void *>(fp8_linear_kernel));
+        if (rc != BONSAI_DECODE_OK) return rc;
     }
     const int nwaves = K % 1024 == 0 ? 8 : (K % 512 == 0 ? 4 : (K % 256 == 0 ? 2 : 1));
     const int ntiles = (N + 15) / 16;

@@ -54,6 +54,8 @@ def load_decode_kernel() -> None:
     lib.bonsai_draft_chain_ws.restype = ci
     lib.bonsai_draft_chain_static.argtypes = [vp, ci, ci, ci, cf, vp, vp, vp, vp]
     lib.bonsai_draft_chain_static.restype = ci
+    lib.bonsai_decode_init.argtypes = []
+    lib.bonsai_decode_init.restype = ci
     lib.bonsai_draft_chain_scratch_bytes.argtypes = [ci]
     lib.bonsai_draft_chain_scratch_bytes.restype = ctypes.c_int64
     lib.bonsai_bf16_linear.argtypes = [vp, vp, vp, ci, ci, ci, vp]

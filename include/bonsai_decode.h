@@ -41,6 +41,8 @@ extern "C" {
 #define BONSAI_DECODE_OK 0
 #define BONSAI_DECODE_ERR_ARG 1
 #define BONSAI_DECODE_ERR_LAUNCH 2
+#define BONSAI_DECODE_ERR_NOT_INIT 3 /* a one-time set-up would have run on a capturing stream:
+                                        call bonsai_decode_init before the capture */
 
 #define BONSAI_HEAD_DIM 128     /* the only head size of the Bonsai/Qwen3 family */
 #define BONSAI_MAX_WIDTH 32     /* rows per step (the reference uses at most 17) */
@@ -126,10 +128,16 @@ int bonsai_draft_chain_ws(const void *logits, int rows, int ld, int vocab, float
  * process ends) instead of a caller workspace; the call allocates and frees nothing.
  * rows <= BONSAI_MAX_WIDTH, larger inputs are refused with BONSAI_DECODE_ERR_ARG.  All calls
  * on one GPU share that array: calls that overlap in time on one GPU (different streams) race.
- * The first call on a device looks the array's address up; make that call outside stream
- * capture. */
+ * The array's address is looked up once per device, by bonsai_decode_init or by the first
+ * call; a first call that arrives on a capturing stream is refused with
+ * BONSAI_DECODE_ERR_NOT_INIT and launches nothing. */
 int bonsai_draft_chain_static(const void *logits, int rows, int ld, int vocab, float threshold,
                               int32_t *tokens, float *conf, int32_t *accept, void *stream);
+
+/* One-time set-up for the current device of what bonsai_draft_chain_static needs (the device
+ * address of the library's scratch array).  Allocates nothing; call it before capturing a graph
+ * whose first launch would be that entry point.  No reference counterpart. */
+int bonsai_decode_init(void);
 
 /* bf16 output projection of a sign-weight (Q1) backbone, whose graphs keep the tied lm_head
  * in bf16: logits = F.linear(h, W) (`_lm_head`, precision "bf16",

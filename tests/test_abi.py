@@ -74,7 +74,7 @@ def test_decode_library_exports_and_binding(libs):
                  "bonsai_bf16_linear", "bonsai_fp8_quant_rows", "bonsai_fp8_linear",
                  "bonsai_decode_set_tuning", "bonsai_decode_set_attention_engine",
                  "bonsai_draft_chain_ws", "bonsai_draft_chain_scratch_bytes",
-                 "bonsai_draft_chain_static"):
+                 "bonsai_draft_chain_static", "bonsai_decode_init"):
         assert name in declared_functions() and hasattr(dec, name)
     from bitmtp_amd import decode_ops
     decode_ops.load_decode_kernel()
