@@ -66,7 +66,7 @@ KERNELS = {"auto": (0, 0), "dot4": (1000, 0), "staged": (1, 1), "operand": (1, 3
 
 
 def sweep(kind: str, shapes, widths, pool_bytes: int = 640 << 20, max_pool: int = 256, seed: int = 4,
-          kernel: str = "auto"):
+          kernel: str = "auto", quiet: bool = False):
     import torch
     import bitmtp_amd as ops
     from bitmtp_amd import ops as ops_mod
@@ -132,8 +132,10 @@ def sweep(kind: str, shapes, widths, pool_bytes: int = 640 << 20, max_pool: int 
                 "us_per_launch": round(best * 1e6, 3),
                 "gbps": round(nbytes / best / 1e9, 1),
                 "pct_hbm_peak": round(nbytes / best / 1e9 / HBM_PEAK_GBPS * 100, 2),
+                "launched": ops_mod.last_kernel(2 if kind == "t2" else 1),
             })
-            print(json.dumps(results[-1]), flush=True)
+            if not quiet:
+                print(json.dumps(results[-1]), flush=True)
         del mats
         torch.cuda.empty_cache()
     (lib.t2g128_set_mfma_tuning if kind == "t2" else lib.q1g128_set_mfma_tuning)(0, 0, 0, 0, 0)
