@@ -411,9 +411,15 @@ def main() -> int:
                     help="comma list restricting the widths measured (profiling runs); default 1,4,8")
     ap.add_argument("--no-drop-in", action="store_true",
                     help="skip the one-launch-per-projection and merged-matrix figures (profiling runs)")
+    ap.add_argument("--kernel-digest", action="store_true",
+                    help="print the digest of the GEMV kernel sources (the key profiles/traffic.json "
+                         "is stored under) and exit; needs no GPU")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device copy (for scaling rocprofv3 PMC byte counters)")
     args = ap.parse_args()
+    if args.kernel_digest:
+        print(kernel_sources_digest())
+        return 0
     global WIDTHS
     if args.widths:
         WIDTHS = tuple(int(w) for w in args.widths.split(","))

@@ -55,9 +55,50 @@ __global__ void __launch_bounds__(256) probe_barrier_kernel(unsigned *state, int
     if (s_bad && threadIdx.x == 0) atomicOr(&state[1], 1u);
 }
 
+// "Last arriver finishes": every workgroup writes a record of `words` 32-bit words (at most 64), makes it visible to the
+// device and bumps an arrival counter; the workgroup that arrives last reads all records (what a
+// fused consumer stage would do), writes one result word and resets the counter.  Nobody waits.
+// mode 0: producers only (records written, no counter); mode 1: with the arrival counter and
+// the finishing stage; mode 2: the finishing stage alone, as the separate launch it would replace.
+__global__ void __launch_bounds__(256) probe_last_arriver_kernel(unsigned *records, unsigned *state,
+                                                               int n_records, int words, int mode) {
+    const unsigned wg = blockIdx.x;
+    __shared__ unsigned s_last;
+    if (mode != 2) {
+        if ((int)threadIdx.x < words) records[wg * words + threadIdx.x] = wg + threadIdx.x;
+        if (mode == 0) return;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            __threadfence();  // the records of this workgroup before its arrival
+            const unsigned old = __hip_atomic_fetch_add(&state[0], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = old == gridDim.x - 1 ? 1u : 0u;
+        }
+        __syncthreads();
+        if (!s_last) return;
+        __threadfence();
+    }
+    unsigned acc = 0;
+    for (int i = threadIdx.x; i < n_records * words; i += 256)
+        acc += records[i];  // ordinary loads: the fence above (mode 1) or the kernel boundary orders them
+    atomicAdd(&state[1], acc);
+    if (threadIdx.x == 0 && mode == 1) __hip_atomic_store(&state[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 }  // namespace
 
 extern "C" {
+
+int bonsai_probe_last_arriver(int launches, int workgroups, int words, int mode, void *records,
+                              void *state, void *stream) {
+    if (launches < 1 || workgroups < 1 || workgroups > 65536 || words < 1 || words > 64 || mode < 0 ||
+        mode > 2 || records == nullptr || state == nullptr)
+        return 1;
+    for (int i = 0; i < launches; ++i)
+        hipLaunchKernelGGL(probe_last_arriver_kernel, dim3(mode == 2 ? 1 : workgroups), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), static_cast<unsigned *>(records),
+                           static_cast<unsigned *>(state), workgroups, words, mode);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
+}
 
 int bonsai_read_probe(const void *src, size_t bytes, int workgroups, int persistent, void *sink,
                       void *stream) {

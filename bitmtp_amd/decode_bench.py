@@ -92,6 +92,68 @@ def run_decode_bench(model_name: str = "1.7b", prompt_len: int = 256, new_tokens
     return res
 
 
+def run_slot_costs(model_name: str = "1.7b", cache_len: int = 500, device: str = "cuda:0",
+                   replays: int = 30) -> dict:
+    """What each operator type costs INSIDE the captured step: the step is captured again with
+    one operator type left out (its launches are simply not enqueued; the results are garbage,
+    only the time counts) and the difference to the complete graph is divided by the launches
+    left out.  Width 1 (role ar) and width 9 (role verify).  Measurement only: the operators
+    are swapped out through this module's own references, nothing in the libraries changes."""
+    from . import decode_ops, model as mdl, ops
+    args = MODELS[model_name]()
+    model = BonsaiDecoder.random_init(args, seed=0, device=device)
+    actq = ops.actq_lib()
+    n_layers = args.n_layers
+
+    class WithoutEntryPoints:
+        """The activation-producer library with chosen entry points turned into no-ops."""
+        def __init__(self, skip):
+            self.skip = skip
+
+        def __getattr__(self, name):
+            return (lambda *a: 0) if name in self.skip else getattr(actq, name)
+
+    def graph_us(M, role):
+        atlas = GraphAtlas(model)
+        sigma = atlas.select_segment(1024)
+        g = atlas.get_graph(M, sigma, role)
+        atlas.replay(g, [1] * M, list(range(cache_len, cache_len + M)), cache_len, 0)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(replays):
+            g.graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / replays * 1e3
+
+    saved = (mdl._gemv, decode_ops.qk_norm_rope_kv_write, decode_ops.decode_attention, ops.actq_lib)
+    out = {"model": model_name, "cache_len": cache_len, "widths": {}}
+    try:
+        for M, role in ((1, "ar"), (9, "verify")):
+            base = graph_us(M, role)
+            row = {"graph_us": round(base, 1), "launches": 10 * n_layers + 4}
+            mdl._gemv = lambda *a, **k: None
+            row["gemv_us_per_launch"] = round((base - graph_us(M, role)) / (4 * n_layers + 1), 2)
+            mdl._gemv = saved[0]
+            decode_ops.qk_norm_rope_kv_write = lambda *a, **k: None
+            row["qk_norm_rope_kv_write_us_per_launch"] = round((base - graph_us(M, role)) / n_layers, 2)
+            decode_ops.qk_norm_rope_kv_write = saved[1]
+            decode_ops.decode_attention = lambda *a, **k: None
+            row["attention_us_per_layer_2_launches"] = round((base - graph_us(M, role)) / n_layers, 2)
+            decode_ops.decode_attention = saved[2]
+            ops.actq_lib = lambda: WithoutEntryPoints({"bonsai_silu_mul_quant_int8"})
+            row["silu_mul_quant_us_per_launch"] = round((base - graph_us(M, role)) / n_layers, 2)
+            ops.actq_lib = lambda: WithoutEntryPoints({"bonsai_add_rmsnorm_quant_int8",
+                                                       "bonsai_rmsnorm_quant_int8"})
+            row["add_norm_quant_us_per_launch"] = round((base - graph_us(M, role)) / (2 * n_layers + 1), 2)
+            ops.actq_lib = saved[3]
+            out["widths"][str(M)] = row
+    finally:
+        mdl._gemv, decode_ops.qk_norm_rope_kv_write, decode_ops.decode_attention, ops.actq_lib = saved
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--model", choices=sorted(MODELS), default="1.7b")
@@ -107,7 +169,13 @@ def main() -> None:
     ap.add_argument("--draft", choices=("native", "fp8", "bf16"), default="native",
                     help="draft output projection: the backbone's own, or the FP8 / raw bf16 "
                          "approximation (verification always uses the backbone's own)")
+    ap.add_argument("--slot-costs", action="store_true",
+                    help="instead of tokens/s: the cost of each operator type inside the captured "
+                         "step (graphs captured with that operator left out)")
     a = ap.parse_args()
+    if a.slot_costs:
+        print(json.dumps(run_slot_costs(a.model)))
+        return
     print(json.dumps(run_decode_bench(a.model, a.prompt, a.new, a.seed, a.repeats,
                                       n_layers=a.layers, kernel_kind=a.kind, head_kind=a.head,
                                       draft_precision=a.draft)))

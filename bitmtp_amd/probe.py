@@ -40,6 +40,8 @@ def probe_lib() -> ctypes.CDLL:
         lib.bonsai_probe_chain_launches.restype = ci
         lib.bonsai_probe_grid_barrier.argtypes = [ci, ci, vp, vp]
         lib.bonsai_probe_grid_barrier.restype = ci
+        lib.bonsai_probe_last_arriver.argtypes = [ci, ci, ci, ci, vp, vp, vp]
+        lib.bonsai_probe_last_arriver.restype = ci
         _lib = lib
     return _lib
 
@@ -141,6 +143,32 @@ def grid_barrier_us(torch, dev, workgroups: int, barriers: int = 101) -> float:
     return (run(barriers) - run(1)) / (barriers - 1)
 
 
+def last_arriver_us(torch, dev, workgroups: int, words: int, launches: int = 500) -> dict:
+    """Microseconds per launch, in one HIP graph of `launches` dependent launches each: producers
+    only, producers with the arrival counter and the finishing stage fused behind it, and the
+    pair (producers, then the finishing stage as a launch of its own)."""
+    lib = probe_lib()
+    records = torch.zeros(workgroups * 64, dtype=torch.int32, device=dev)
+    state = torch.zeros(2, dtype=torch.int32, device=dev)
+    out = {}
+    for name, modes in (("producers_only", (0,)), ("fused_last_arriver", (1,)), ("two_launches", (0, 2))):
+        def enqueue(sp, modes=modes):
+            for _ in range(launches):
+                for mode in modes:
+                    rc = lib.bonsai_probe_last_arriver(1, workgroups, words, mode, records.data_ptr(),
+                                                       state.data_ptr(), sp)
+                    if rc != 0:
+                        raise RuntimeError(f"bonsai_probe_last_arriver returned {rc}")
+        state.zero_()
+        enqueue(_stream_ptr(torch))
+        torch.cuda.synchronize()
+        state.zero_()
+        g = _graph_of(torch, enqueue)
+        out[name] = _time_us(torch, g.replay) / launches
+        del g
+    return out
+
+
 def main() -> int:
     import torch
     if not torch.cuda.is_available():
@@ -168,6 +196,10 @@ def main() -> int:
     emit("read_stream", bytes=head, workgroups=512, us=read_probe_us(torch, head, 512, True, dev))
     for wgs in (256, 512, 1024):
         emit("grid_barrier", workgroups=wgs, us_per_barrier=grid_barrier_us(torch, dev, wgs))
+    # o / down projection of the 1.7B layer: 128 row tiles of 16 rows; one token is 8 words (16
+    # bf16) per workgroup, nine tokens 64+ (capped)
+    for wgs, words in ((128, 8), (128, 64), (768, 8)):
+        emit("last_arriver", workgroups=wgs, words_per_record=words, **last_arriver_us(torch, dev, wgs, words))
     return 0
 
 

@@ -43,6 +43,18 @@ int bonsai_probe_chain_launches(int launches, void *word, void *stream);
  * kernel always ends). */
 int bonsai_probe_grid_barrier(int workgroups, int barriers, void *state, void *stream);
 
+/* Enqueues `launches` launches of the "last arriver finishes" probe over `workgroups` workgroups
+ * of 256 threads.  mode 0: every workgroup writes a record of `words` (1..64) 32-bit words and
+ * ends; mode 1: it then
+ * makes the record visible, bumps an arrival counter, and the workgroup that arrives last reads
+ * all records, adds them into state[1] and resets the counter (no workgroup ever waits); mode 2:
+ * one workgroup that only reads the records -- the separate launch that mode 1 would save.
+ * `records` holds workgroups x words words, `state` two zeroed words.  time(mode 1) against
+ * time(mode 0) + time(mode 2) is what fusing a consumer stage behind an arrival counter gains or
+ * loses over launching it on its own. */
+int bonsai_probe_last_arriver(int launches, int workgroups, int words, int mode, void *records,
+                              void *state, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
