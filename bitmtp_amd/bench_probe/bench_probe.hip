@@ -80,7 +80,8 @@ __global__ void __launch_bounds__(256) probe_last_arriver_kernel(unsigned *recor
     unsigned acc = 0;
     for (int i = threadIdx.x; i < n_records * words; i += 256)
         acc += records[i];  // ordinary loads: the fence above (mode 1) or the kernel boundary orders them
-    atomicAdd(&state[1], acc);
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+    if ((threadIdx.x & 63) == 0) atomicAdd(&state[1], acc);  // one result word per wave
     if (threadIdx.x == 0 && mode == 1) __hip_atomic_store(&state[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
