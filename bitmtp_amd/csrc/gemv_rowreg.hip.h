@@ -43,25 +43,6 @@ struct RowregParams {
 
 constexpr int kRowregBufferWord3 = 0x00020000;  // raw buffer, 32-bit format, range check on
 
-// Sixteen natural-order activations (four dwords) -> {even hi, even lo, odd hi, odd lo}: nibble
-// n of an "even" word belongs to activation 2 n, of an "odd" word to activation 2 n + 1; hi is
-// the signed upper and lo the unsigned lower four bits.
-__device__ __forceinline__ u32x4 nibble_planes16(const u32x4 in) {
-    const uint32_t e0 = __builtin_amdgcn_perm(in.y, in.x, 0x06040200u);
-    const uint32_t e1 = __builtin_amdgcn_perm(in.w, in.z, 0x06040200u);
-    const uint32_t o0 = __builtin_amdgcn_perm(in.y, in.x, 0x07050301u);
-    const uint32_t o1 = __builtin_amdgcn_perm(in.w, in.z, 0x07050301u);
-    const auto lo = [](uint32_t x) { return x & 0x0f0f0f0fu; };
-    const auto hi = [](uint32_t x) { return (x >> 4) & 0x0f0f0f0fu; };
-    const auto pk = [](uint32_t x) { return x | (x >> 4); };  // bytes 0 and 2: two nibbles each
-    u32x4 r;
-    r.x = __builtin_amdgcn_perm(pk(hi(e1)), pk(hi(e0)), 0x06040200u);
-    r.y = __builtin_amdgcn_perm(pk(lo(e1)), pk(lo(e0)), 0x06040200u);
-    r.z = __builtin_amdgcn_perm(pk(hi(o1)), pk(hi(o0)), 0x06040200u);
-    r.w = __builtin_amdgcn_perm(pk(lo(o1)), pk(lo(o0)), 0x06040200u);
-    return r;
-}
-
 // G32: store the exact int32 group sums G[0][n][g] instead of the scaled result.
 template <int LPR_LOG2, bool SF16, bool G32 = false>
 __global__ void __launch_bounds__(kRowregThreads) __attribute__((amdgpu_waves_per_eu(4)))

@@ -36,6 +36,10 @@ namespace bonsai {
 constexpr int kGroup = 128;
 constexpr int kMaxTile = 8;       // tokens per tile (template MT is 1..kMaxTile)
 constexpr int kMaxThreads = 512;  // workgroup size limit of the kernels
+#ifndef BONSAI_PLANE_MAX_TILE
+#define BONSAI_PLANE_MAX_TILE 2
+#endif
+constexpr int kPlaneMaxTile = BONSAI_PLANE_MAX_TILE;  // widest T2 token tile that takes the 4-bit-plane form
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_G32 = 2 };
 
@@ -136,6 +140,68 @@ struct WeightBatch {
     uint16_t sraw[U];
 };
 
+// ---- 4-bit planes (T2, narrow token tiles) -------------------------------------------------
+// For one or two tokens the dot4 body is bound by its vector instructions (seven to unpack a
+// packed dword into byte vectors, four v_dot4 per token).  With the activations staged as 4-bit
+// planes, a = 16 hi + lo (hi signed, lo unsigned; even and odd positions apart), the codes are
+// only masked to nibbles -- e = p & 0x33333333, o = (p >> 2) & 0x33333333: three operations --
+// and meet the planes in four v_dot8 per token: 28 operations per 16-byte chunk against 44.
+// raw = 16 H + L is the same integer sum of a * code the byte form gives.
+
+// Sixteen natural-order activations (four dwords) -> {even hi, even lo, odd hi, odd lo}: nibble
+// n of an "even" word belongs to activation 2 n, of an "odd" word to activation 2 n + 1.
+__device__ __forceinline__ u32x4 nibble_planes16(const u32x4 in) {
+    const uint32_t e0 = __builtin_amdgcn_perm(in.y, in.x, 0x06040200u);
+    const uint32_t e1 = __builtin_amdgcn_perm(in.w, in.z, 0x06040200u);
+    const uint32_t o0 = __builtin_amdgcn_perm(in.y, in.x, 0x07050301u);
+    const uint32_t o1 = __builtin_amdgcn_perm(in.w, in.z, 0x07050301u);
+    const auto lo = [](uint32_t x) { return x & 0x0f0f0f0fu; };
+    const auto hi = [](uint32_t x) { return (x >> 4) & 0x0f0f0f0fu; };
+    const auto pk = [](uint32_t x) { return x | (x >> 4); };  // bytes 0 and 2: two nibbles each
+    u32x4 r;
+    r.x = __builtin_amdgcn_perm(pk(hi(e1)), pk(hi(e0)), 0x06040200u);
+    r.y = __builtin_amdgcn_perm(pk(lo(e1)), pk(lo(e0)), 0x06040200u);
+    r.z = __builtin_amdgcn_perm(pk(hi(o1)), pk(hi(o0)), 0x06040200u);
+    r.w = __builtin_amdgcn_perm(pk(lo(o1)), pk(lo(o0)), 0x06040200u);
+    return r;
+}
+
+// Plane form of stage_quarter<2, MT>: the same LDS slot receives the four plane words of the
+// quarter's sixteen activations; returns their sum.
+template <int MT>
+__device__ __forceinline__ int stage_quarter_planes(const u32x4 *src, u32x4 *act, int m, int chunk, int sub) {
+    const u32x4 in = src[0];
+    act[act_index<2, MT>(m, sub, chunk)] = nibble_planes16(in);
+    return sum4_i8(in.x) + sum4_i8(in.y) + sum4_i8(in.z) + sum4_i8(in.w);
+}
+
+// Plane form of chunk_dot_raw<2, MT>: raw[m] += sum a[m][k] * code[k] over the chunk.
+template <int MT>
+__device__ __forceinline__ void chunk_dot_raw_planes(const u32x4 w, const u32x4 *act, int chunk, int raw[MT]) {
+    const uint32_t p[4] = {w.x, w.y, w.z, w.w};
+    int ah[MT];
+    uint32_t al[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        ah[m] = 0;
+        al[m] = 0;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const uint32_t e = p[t] & 0x33333333u, o = (p[t] >> 2) & 0x33333333u;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const u32x4 a = act[act_index<2, MT>(m, t, chunk)];
+            ah[m] = __builtin_amdgcn_sdot8((int)a.x, (int)e, ah[m], false);
+            al[m] = __builtin_amdgcn_udot8(a.y, e, al[m], false);
+            ah[m] = __builtin_amdgcn_sdot8((int)a.z, (int)o, ah[m], false);
+            al[m] = __builtin_amdgcn_udot8(a.w, o, al[m], false);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) raw[m] += (ah[m] << 4) + (int)al[m];
+}
+
 // BITS: 2 = T2, 1 = Q1.  MT: tokens in the tile.  U: 16-byte weight loads a lane
 // issues back to back (one batch).  G32: write the int32 group sums instead of
 // the scaled result.  SF16: group scales are fp16 instead of bf16.
@@ -144,6 +210,8 @@ template <int BITS, int MT, int U, bool G32, bool SF16>
 __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by, int pthreads,
                                                unsigned char *smem) {
     using F = Fmt<BITS>;
+    // 4-bit planes and v_dot8 for T2 tiles of one or two tokens (see above)
+    constexpr bool P4 = BITS == 2 && MT <= kPlaneMaxTile;
 
     const int K = a.K, N = a.N, M = a.M;
     const int C = K / F::kChunkWeights;  // 16-byte chunks per weight row
@@ -216,7 +284,11 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
 
     // ---- stage the token tile: permuted activations and per-chunk sums into LDS
     if (has_first) {
-        int qs = stage_quarter<BITS, MT>(first_q, act, fm, fchunk, fsub);
+        int qs;
+        if constexpr (P4)
+            qs = stage_quarter_planes<MT>(first_q, act, fm, fchunk, fsub);
+        else
+            qs = stage_quarter<BITS, MT>(first_q, act, fm, fchunk, fsub);
         qs += dpp_i32<kDppXor1>(qs);
         qs += dpp_i32<kDppXor2>(qs);
         if (fsub == 0) asum[asum_index<BITS, MT>(fm, fchunk)] = qs;
@@ -224,7 +296,11 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
     for (int task = tid + nthreads; task < ntasks; task += nthreads) {
         int m, chunk, sub;
         const u32x4 *src = task_src(task, m, chunk, sub);
-        int qs = stage_quarter<BITS, MT>(src, act, m, chunk, sub);
+        int qs;
+        if constexpr (P4)
+            qs = stage_quarter_planes<MT>(src, act, m, chunk, sub);
+        else
+            qs = stage_quarter<BITS, MT>(src, act, m, chunk, sub);
         qs += dpp_i32<kDppXor1>(qs);
         qs += dpp_i32<kDppXor2>(qs);
         if (sub == 0) asum[asum_index<BITS, MT>(m, chunk)] = qs;
@@ -248,7 +324,10 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
             int raw[MT];
 #pragma unroll
             for (int m = 0; m < MT; ++m) raw[m] = 0;
-            chunk_dot_raw<BITS, MT>(wb.w[u], act, chunk_c, raw);
+            if constexpr (P4)
+                chunk_dot_raw_planes<MT>(wb.w[u], act, chunk_c, raw);
+            else
+                chunk_dot_raw<BITS, MT>(wb.w[u], act, chunk_c, raw);
             float wsf = 0.0f;
             if (!G32) wsf = scale_to_f32<SF16>(wb.sraw[u]);
 #pragma unroll
