@@ -71,10 +71,12 @@ def test_default_kernels_do_not_spill(reports, bits):
 def test_lean_kernel_residency(reports, bits):
     """Blocks of at most eight tokens (NB = 1, four waves per workgroup) leave room for five waves
     per SIMD, which is what makes the 1280 workgroups of a layer-sized launch resident at once."""
-    rep = _select(reports[bits], rf"gemv_mxl_kernel<{bits}, 4, (true|false), 4, 1, 5>")
+    # (the last template argument is the output kind: false = scaled result, true = group sums)
+    rep = _select(reports[bits], rf"gemv_mxl_kernel<{bits}, 4, (true|false), 4, 1, 5, false>")
     assert len(rep) == 2
     for name, v in rep.items():
         assert v["occupancy"] >= 5 and v["vgprs"] <= 96, (name, v)
-    five_wave_two_batch = _select(reports[bits], rf"gemv_mxl_kernel<{bits}, 4, (true|false), 4, 2, 5>")
+    five_wave_two_batch = _select(reports[bits], rf"gemv_mxl_kernel<{bits}, 4, (true|false), 4, 2, 5, (true|false)>")
+    assert len(five_wave_two_batch) == 3
     for name, v in five_wave_two_batch.items():
         assert v["occupancy"] >= 5 and v["scratch"] == 0, (name, v)
