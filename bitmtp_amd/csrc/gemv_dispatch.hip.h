@@ -425,6 +425,67 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
                                   stream);
 }
 
+// ---- the MLP tail as two launches (blocks of one or two tokens; see packed_gemv.hip.h) ------
+constexpr int kFusedMaxWidth = kFusedMaxTile;
+
+template <int BITS>
+int fused_ready(int M, int N, int K, hipStream_t stream, int *lds_limit) {
+    if (M < 1 || M > kFusedMaxWidth || N < 1 || K < kGroup || K % kGroup != 0) return 1;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 2;
+    const int rc = ensure_ready<BITS>(dev, stream);
+    if (rc != 0) return rc;
+    *lds_limit = lib_state<BITS>().lds_limit[dev];
+    return 0;
+}
+
+// Parts per token that launch_gemv_silu_pair writes for this shape (its workgroup count), or a
+// negative status: -1 the shape is not taken, -2 / -3 as the launch statuses 2 / 3.
+template <int BITS>
+int silu_pair_parts(int M, int N2, int K) {
+    if (N2 < 2 || (N2 & 1)) return -1;
+    int lds_limit = 0;
+    const int rc = fused_ready<BITS>(M, N2, K, nullptr, &lds_limit);
+    if (rc != 0) return -rc;
+    const Geometry g = fused_geometry<BITS>(FUSE_SILU_PAIR, M, N2, K, lds_limit);
+    return g.mt == 0 ? -1 : g.grid_x;
+}
+
+// gate|up projection (rows [gate; up], N2 = 2 F of them) of int8 activations: writes
+// inner = bf16(bf16(silu(gate)) * up) as bf16 [M, F] and max |inner| per token and workgroup
+// into `amax` (bf16 [M, amax_ld(parts)], parts = silu_pair_parts(M, N2, K); every element is written).
+template <int BITS>
+int launch_gemv_silu_pair(const int8_t *A, const uint8_t *B, void *inner, const float *s, const void *ws,
+                          int M, int N2, int K, uint16_t *amax, hipStream_t stream) {
+    if (A == nullptr || B == nullptr || inner == nullptr || s == nullptr || ws == nullptr || amax == nullptr)
+        return 1;
+    if (N2 < 2 || (N2 & 1)) return 1;
+    if (!operands_aligned(A, B, inner, s, ws, OUT_BF16) || (reinterpret_cast<uintptr_t>(amax) & 15)) return 1;
+    int lds_limit = 0;
+    const int rc = fused_ready<BITS>(M, N2, K, stream, &lds_limit);
+    if (rc != 0) return rc;
+    return launch_gemv_dot4_fused<BITS>(FUSE_SILU_PAIR, A, B, inner, s, ws, M, N2, K, OUT_BF16, amax, 0,
+                                        nullptr, lds_limit, stream);
+}
+
+// Down projection of `inner` (bf16 [M, K]) quantised on the fly with the multiplier derived from
+// the `parts` maxima per token in `amax`; writes the multipliers to `s_out` when that is given.
+template <int BITS>
+int launch_gemv_bf16_act(const void *inner, const uint8_t *B, void *out, const void *ws, int M, int N,
+                         int K, const uint16_t *amax, int parts, float *s_out, int out_kind,
+                         hipStream_t stream) {
+    if (inner == nullptr || B == nullptr || out == nullptr || ws == nullptr || amax == nullptr) return 1;
+    if (out_kind != OUT_BF16 && out_kind != OUT_F32) return 1;
+    if (parts < 1 || parts > kAmaxMaxParts) return 1;
+    if (!operands_aligned(inner, B, out, s_out, ws, out_kind) || (reinterpret_cast<uintptr_t>(amax) & 15))
+        return 1;
+    int lds_limit = 0;
+    const int rc = fused_ready<BITS>(M, N, K, stream, &lds_limit);
+    if (rc != 0) return rc;
+    return launch_gemv_dot4_fused<BITS>(FUSE_BF16_ACT, inner, B, out, nullptr, ws, M, N, K, out_kind,
+                                        const_cast<uint16_t *>(amax), parts, s_out, lds_limit, stream);
+}
+
 // Several GEMVs in one call (descriptors in host memory, read before the call returns).
 // Problems the grouped kernel takes (K % 512 == 0, aligned operands) share launches of up to
 // kMxMaxDesc descriptors each, blocks wider than 16 tokens as several token tiles; the rest

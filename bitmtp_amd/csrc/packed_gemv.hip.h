@@ -30,6 +30,7 @@
 #include <stdio.h>
 
 #include "gemv_core.h"
+#include "wave_reduce.h"
 
 namespace bonsai {
 
@@ -91,7 +92,61 @@ struct GemvArgs {
     int passes;          // row passes per wave
     int out_f32;         // 1: store the fp32 value, 0: round to bf16
     uint32_t div_magic;  // floor(2^32 / (4*C)) + 1, for task -> token in the staging loop
+    uint16_t *amax = nullptr;       // FUSE_SILU_PAIR: receives, FUSE_BF16_ACT: holds max |inner| (bf16) per token and part
+    int amax_parts = 0;             // parts per token: the workgroup count of the FUSE_SILU_PAIR launch
+    float *s_out = nullptr;         // FUSE_BF16_ACT: receives the multipliers (may be null)
 };
+
+// ---- the MLP tail without its middle launch ------------------------------------------------
+// Between the gate|up projection and the down projection the reference runs one fused Python
+// helper (src/bonsai_sft/gpu/model.py:1059-1061): inner = bf16(bf16(silu(gate)) * up), then
+// the per-token absmax quantisation of inner.  For blocks of one or two tokens that launch
+// costs as much as either projection.  Two forms of the dot4 kernel take its place:
+//   FUSE_SILU_PAIR  the gate|up projection visits its rows in the order gate 0, up 0, gate 1,
+//                   up 1, ... so that the two results of a column meet in neighbouring lane
+//                   sets; it writes inner (bf16, [M, N/2]) and, per workgroup and token, max |inner|
+//                   of what the workgroup stored (its waves meet in LDS; plain stores, no atomics
+//                   in memory -- 1536 atomic maxima spread over 32 cache lines cost 0.9 us on a
+//                   3.5 us launch, on two lines 13 us);
+//   FUSE_BF16_ACT   the down projection reads inner and the parts, derives the multiplier
+//                   s = fl(fl(1 / max(amax, 1e-5)) * 127) and quantises each value while it stages
+//                   it: q = clamp(rne(fl(x * s)), -128, 127).
+// Same operations on the same values as the three-launch form, so the results are the same bits.
+constexpr int FUSE_NONE = 0, FUSE_SILU_PAIR = 1, FUSE_BF16_ACT = 2;
+// The parts are bf16 (max |inner| is one of the bf16 values stored): up to 1024 of them are two
+// 16-byte loads per lane of a wave.
+constexpr int kAmaxMaxParts = 1024;
+// elements per token of the parts array: parts rounded up to whole 16-byte words (the pad holds 0)
+__host__ __device__ constexpr int amax_ld(int parts) { return (parts + 7) & ~7; }
+
+__device__ __forceinline__ float bf16_round_f32(float f) {
+    const __bf16 b = static_cast<__bf16>(f);  // round to nearest even (v_cvt_pk_bf16_f32)
+    uint16_t u;
+    __builtin_memcpy(&u, &b, 2);
+    return __uint_as_float((uint32_t)u << 16);
+}
+
+// bf16(bf16(silu(g)) * u) with silu through the hardware exp2 and reciprocal, exactly as
+// silu_mul_quant_kernel (act_quant.hip) evaluates it.
+__device__ __forceinline__ float silu_mul_bf16(float g, float u) {
+    const float ex = __builtin_amdgcn_exp2f(g * -1.44269504088896341f);
+    const float sg = bf16_round_f32(g * __builtin_amdgcn_rcpf(1.0f + ex));
+    return bf16_round_f32(sg * u);
+}
+
+// Sixteen bf16 values (two 16-byte words) -> sixteen int8 in natural order.
+__device__ __forceinline__ u32x4 quant16_bf16(const u32x4 lo, const u32x4 hi, float s) {
+    const auto q1 = [s](uint32_t bits) {
+        float r = __builtin_rintf(__uint_as_float(bits) * s);
+        r = fminf(fmaxf(r, -128.0f), 127.0f);
+        return (uint32_t)((int)r) & 0xffu;
+    };
+    const auto q4 = [&q1](uint32_t d0, uint32_t d1) {
+        return q1(d0 << 16) | (q1(d0 & 0xffff0000u) << 8) | (q1(d1 << 16) << 16) |
+               (q1(d1 & 0xffff0000u) << 24);
+    };
+    return u32x4{q4(lo.x, lo.y), q4(lo.z, lo.w), q4(hi.x, hi.y), q4(hi.z, hi.w)};
+}
 
 template <bool SF16>
 __device__ __forceinline__ float scale_to_f32(uint16_t raw) {
@@ -206,10 +261,11 @@ __device__ __forceinline__ void chunk_dot_raw_planes(const u32x4 w, const u32x4 
 // issues back to back (one batch).  G32: write the int32 group sums instead of
 // the scaled result.  SF16: group scales are fp16 instead of bf16.
 // The kernel proper: workgroup `bx` of the GEMV `a`, token tile `by`, `pthreads` threads.
-template <int BITS, int MT, int U, bool G32, bool SF16>
+template <int BITS, int MT, int U, bool G32, bool SF16, int FUSE = FUSE_NONE>
 __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by, int pthreads,
                                                unsigned char *smem) {
     using F = Fmt<BITS>;
+    static_assert(FUSE == FUSE_NONE || (!G32 && MT <= 2), "fused forms: one or two tokens, scaled output");
     // 4-bit planes and v_dot8 for T2 tiles of one or two tokens (see above)
     constexpr bool P4 = BITS == 2 && MT <= kPlaneMaxTile;
 
@@ -238,8 +294,13 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
 
     // All loads of a batch are unconditional (indices clamped into the row) and
     // issued back to back; lanes past the end of a row are masked when used.
+    // FUSE_SILU_PAIR: visiting order gate 0, up 0, gate 1, up 1, ... over the rows [gate; up]
+    const int half_n = N >> 1;
+    auto stored_row = [&](int row) {
+        return FUSE == FUSE_SILU_PAIR ? (row & 1) * half_n + (row >> 1) : row;
+    };
     auto load_batch = [&](WeightBatch<U> &wb, int row, int it0) {
-        const int row_c = row < N ? row : N - 1;
+        const int row_c = stored_row(row < N ? row : N - 1);
         const u32x4 *wrow = reinterpret_cast<const u32x4 *>(a.B) + (size_t)row_c * C;
         const uint16_t *srow = a.ws + (size_t)row_c * ng;
 #pragma unroll
@@ -255,40 +316,96 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
     // staging data (an L2 hit) is back before the weights (HBM) are.
     const int ntasks = MT * C * 4;  // quarter chunks to stage
     constexpr int kQ = F::kUnits / 4;  // 16-byte words per quarter
+    // (FUSE_BF16_ACT: a.A holds bf16 values, twice the bytes per quarter)
+    constexpr int kSrcWords = FUSE == FUSE_BF16_ACT ? 2 * kQ : kQ;
     auto task_src = [&](int task, int &m, int &chunk, int &sub) {
-        m = (int)__umulhi((uint32_t)task, a.div_magic);  // task / (4*C)
+        if constexpr (FUSE != FUSE_NONE)
+            m = (MT > 1 && task >= 4 * C) ? 1 : 0;  // at most two tokens: no division
+        else
+            m = (int)__umulhi((uint32_t)task, a.div_magic);  // task / (4*C)
         const int rest = task - m * 4 * C;
         chunk = rest >> 2;
         sub = rest & 3;
         const int msrc = (m0 + m) < M ? (m0 + m) : M - 1;
-        return reinterpret_cast<const u32x4 *>(a.A + (size_t)msrc * K) +
-               ((size_t)chunk * 4 + sub) * kQ;
+        return reinterpret_cast<const u32x4 *>(a.A + (size_t)msrc * K * (FUSE == FUSE_BF16_ACT ? 2 : 1)) +
+               ((size_t)chunk * 4 + sub) * kSrcWords;
     };
-    u32x4 first_q[kQ];
+    u32x4 first_q[kSrcWords];
     int fm = 0, fchunk = 0, fsub = 0;
     const bool has_first = tid < ntasks;
     if (has_first) {
         const u32x4 *src = task_src(tid, fm, fchunk, fsub);
 #pragma unroll
-        for (int i = 0; i < kQ; ++i) first_q[i] = src[i];
+        for (int i = 0; i < kSrcWords; ++i) first_q[i] = src[i];
+    }
+    // FUSE_BF16_ACT: every wave reads the parts of a token itself, one 16-byte word per lane (a
+    // second workgroup barrier ahead of the staging costs more than the repeated reads)
+    u32x4 part_bits[MT][2];
+    if (FUSE == FUSE_BF16_ACT) {
+        const int words = amax_ld(a.amax_parts) >> 3;  // at most 128
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const u32x4 *prow = reinterpret_cast<const u32x4 *>(
+                a.amax + (size_t)((m0 + m) < M ? (m0 + m) : M - 1) * (words * 8));
+            part_bits[m][0] = prow[lane < words ? lane : words - 1];  // past the end: a repeat
+            part_bits[m][1] = prow[lane + 64 < words ? lane + 64 : words - 1];
+        }
     }
 
     WeightBatch<U> cur, nxt;
     load_batch(cur, row0, 0);
+    if (FUSE == FUSE_SILU_PAIR) asm volatile("" ::"s"(a.amax));  // fetched now, used at the very end
 
     float sdiv[MT];
-    if (!G32) {
+    if (FUSE == FUSE_BF16_ACT) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            // non-negative bf16 values order as unsigned 16-bit integers
+            typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+            const auto pk = [](uint32_t x) { us2 r; __builtin_memcpy(&r, &x, 4); return r; };
+            const u32x4 v = part_bits[m][0], v1 = part_bits[m][1];
+            const us2 p2 = __builtin_elementwise_max(
+                __builtin_elementwise_max(__builtin_elementwise_max(pk(v.x), pk(v.y)),
+                                          __builtin_elementwise_max(pk(v.z), pk(v.w))),
+                __builtin_elementwise_max(__builtin_elementwise_max(pk(v1.x), pk(v1.y)),
+                                          __builtin_elementwise_max(pk(v1.z), pk(v1.w))));
+            const uint32_t top = p2.x > p2.y ? p2.x : p2.y;
+            const float amax = bonsai_wave::max64(__uint_as_float(top << 16));
+            const float recip = 1.0f / fmaxf(amax, 1e-5f);  // IEEE division, rounded on its own
+            sdiv[m] = recip * 127.0f;
+        }
+        if (bx == 0 && wave == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if ((m0 + m) < M && a.s_out != nullptr && lane == 0) a.s_out[m0 + m] = sdiv[m];
+            }
+        }
+    } else if (!G32) {
 #pragma unroll
         for (int m = 0; m < MT; ++m) sdiv[m] = a.s[(m0 + m) < M ? (m0 + m) : M - 1];
     }
+    // FUSE_BF16_ACT: the quarter as int8, quantised with its token's multiplier
+    auto quantised = [&](const u32x4 *raw, int m, u32x4 *q) {
+        float sm = sdiv[0];
+#pragma unroll
+        for (int t = 1; t < MT; ++t) sm = (m == t) ? sdiv[t] : sm;
+#pragma unroll
+        for (int i = 0; i < kQ; ++i) q[i] = quant16_bf16(raw[2 * i], raw[2 * i + 1], sm);
+    };
 
     // ---- stage the token tile: permuted activations and per-chunk sums into LDS
     if (has_first) {
+        u32x4 fq[kQ];
+        const u32x4 *fsrc = first_q;
+        if constexpr (FUSE == FUSE_BF16_ACT) {
+            quantised(first_q, fm, fq);
+            fsrc = fq;
+        }
         int qs;
         if constexpr (P4)
-            qs = stage_quarter_planes<MT>(first_q, act, fm, fchunk, fsub);
+            qs = stage_quarter_planes<MT>(fsrc, act, fm, fchunk, fsub);
         else
-            qs = stage_quarter<BITS, MT>(first_q, act, fm, fchunk, fsub);
+            qs = stage_quarter<BITS, MT>(fsrc, act, fm, fchunk, fsub);
         qs += dpp_i32<kDppXor1>(qs);
         qs += dpp_i32<kDppXor2>(qs);
         if (fsub == 0) asum[asum_index<BITS, MT>(fm, fchunk)] = qs;
@@ -296,6 +413,14 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
     for (int task = tid + nthreads; task < ntasks; task += nthreads) {
         int m, chunk, sub;
         const u32x4 *src = task_src(task, m, chunk, sub);
+        u32x4 tq[kQ];
+        if constexpr (FUSE == FUSE_BF16_ACT) {
+            u32x4 raw[kSrcWords];
+#pragma unroll
+            for (int i = 0; i < kSrcWords; ++i) raw[i] = src[i];
+            quantised(raw, m, tq);
+            src = tq;
+        }
         int qs;
         if constexpr (P4)
             qs = stage_quarter_planes<MT>(src, act, m, chunk, sub);
@@ -305,11 +430,18 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
         qs += dpp_i32<kDppXor2>(qs);
         if (sub == 0) asum[asum_index<BITS, MT>(m, chunk)] = qs;
     }
+    // FUSE_SILU_PAIR: where the waves of the workgroup meet at the end, behind the staged
+    // activations: MT maxima per wave
+    uint32_t *meet = reinterpret_cast<uint32_t *>(smem + (size_t)C * block_words<BITS, MT>() * 16);
     __syncthreads();
 
     float accf[MT];
+    float inner_max[MT];  // FUSE_SILU_PAIR: max |inner| this lane has stored
 #pragma unroll
-    for (int m = 0; m < MT; ++m) accf[m] = 0.0f;
+    for (int m = 0; m < MT; ++m) {
+        accf[m] = 0.0f;
+        inner_max[m] = 0.0f;
+    }
 
     // One batch of one pass: unpack, dot, scale, and after the last batch of the
     // pass reduce over the row's lanes and store.
@@ -352,6 +484,19 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
             for (int m = 0; m < MT; ++m) {
                 const float sum = row_lanes_sum(accf[m], lpr_log2);
                 accf[m] = 0.0f;
+                if constexpr (FUSE == FUSE_SILU_PAIR) {
+                    // every lane of a row's set holds the row's value; the next set (row ^ 1)
+                    // holds the other half of the column
+                    const float mine = bf16_round_f32(sum / sdiv[m]);
+                    const float other = __shfl_xor(mine, lpr);
+                    if (c == 0 && (row & 1) == 0 && row_ok && (m0 + m) < M) {
+                        const float inner = silu_mul_bf16(mine, other);
+                        reinterpret_cast<uint16_t *>(a.out)[(size_t)(m0 + m) * half_n + (row >> 1)] =
+                            (uint16_t)(__float_as_uint(inner) >> 16);
+                        inner_max[m] = fmaxf(inner_max[m], fabsf(inner));
+                    }
+                    continue;
+                }
                 if (c == 0 && row_ok && (m0 + m) < M) {
                     const float y = sum / sdiv[m];
                     if (a.out_f32)
@@ -398,6 +543,39 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
     } else {
         compute_batch(cur, pa, ba);
     }
+    if constexpr (FUSE == FUSE_SILU_PAIR) {
+        // the waves' maxima meet in LDS behind a barrier (every wave is at its end by then) and
+        // thread 0 stores the workgroup's part.  Measured on 12288 x 2048 at one token (3.45 us as
+        // a plain GEMV, 3.70 us with the pairing and SiLU alone): this barrier 3.97 us, a count in
+        // LDS whose last arriver stores 4.14 us, one part per wave 3.83 us (but four times the
+        // parts for every wave of the consumer to read)
+        constexpr int kW = kMaxThreads / 64;
+        float wmax[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) wmax[m] = bonsai_wave::max64(inner_max[m]);
+        if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) meet[m * kW + wave] = __float_as_uint(wmax[m]);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            const int parts = a.amax_parts, ld = amax_ld(parts);  // (the grid size, as a parameter)
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if ((m0 + m) >= M) continue;
+                uint32_t top = 0u;  // non-negative floats order as their bits
+#pragma unroll
+                for (int w = 0; w < kW; ++w) {
+                    const uint32_t v = meet[m * kW + (w < nwaves ? w : nwaves - 1)];
+                    top = v > top ? v : top;
+                }
+                uint16_t *prow = a.amax + (size_t)(m0 + m) * ld;
+                prow[bx] = (uint16_t)(top >> 16);  // exact: one of the bf16 values stored
+                if (bx == parts - 1)
+                    for (int w = parts; w < ld; ++w) prow[w] = 0;
+            }
+        }
+    }
 }
 
 template <int BITS, int MT, int U, bool G32, bool SF16>
@@ -409,6 +587,30 @@ gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *p
     const GemvArgs a{pA, pB, pout, ps, pws, pM, pN, pK, plpr_log2, ppasses, pout_f32, pdiv_magic};
     extern __shared__ __align__(16) unsigned char smem[];
     gemv_dot4_body<BITS, MT, U, G32, SF16>(a, (int)blockIdx.x, (int)blockIdx.y, pthreads, smem);
+}
+
+// The fused forms (FUSE_SILU_PAIR, FUSE_BF16_ACT) of the same body; bf16 scales, bf16 or fp32 out.
+// Sixteen dwords of arguments arrive in SGPRs with the wave; a later one is a scalar load that
+// the compiler places where the value is first needed.  So `px` is what the prologue needs (the
+// multipliers for FUSE_SILU_PAIR, the parts for FUSE_BF16_ACT) and `py` what only the end of the
+// kernel needs (the parts to write / the optional multiplier output); the body asks for `py` once
+// its first loads are on their way.  pgeom = lpr_log2 | passes << 8 | out_f32 << 16.
+template <int BITS, int MT, int U, int FUSE>
+__global__ void __launch_bounds__(kMaxThreads)
+gemv_dot4_fused_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const void *px,
+                       const uint16_t *pws, int pM, int pN, int pK, int pgeom, int pparts,
+                       int pthreads, void *py) {
+    GemvArgs a{pA, pB, pout, nullptr, pws, pM, pN, pK, pgeom & 0xff, (pgeom >> 8) & 0xff, (pgeom >> 16) & 1, 0u};
+    if (FUSE == FUSE_SILU_PAIR) {
+        a.s = static_cast<const float *>(px);
+        a.amax = static_cast<uint16_t *>(py);
+    } else {
+        a.amax = const_cast<uint16_t *>(static_cast<const uint16_t *>(px));
+        a.s_out = static_cast<float *>(py);
+    }
+    a.amax_parts = pparts;
+    extern __shared__ __align__(16) unsigned char smem[];
+    gemv_dot4_body<BITS, MT, U, false, false, FUSE>(a, (int)blockIdx.x, (int)blockIdx.y, pthreads, smem);
 }
 
 // ---- several GEMVs in one launch -------------------------------------------------------
@@ -529,6 +731,9 @@ LibState<BITS> &lib_state() {
     return st;
 }
 
+template <int BITS>
+int init_fused_kernels(int max_lds);
+
 // Raises the dynamic-LDS limit of every kernel instantiation on the current
 // device to what the device offers (160 KB per workgroup on gfx950).
 template <int BITS>
@@ -550,6 +755,7 @@ int init_device() {
                                         hipFuncAttributeMaxDynamicSharedMemorySize,
                                         max_lds) != hipSuccess)
                     return 2;
+    if (init_fused_kernels<BITS>(max_lds) != 0) return 2;
     st.lds_limit[dev] = max_lds;
     return 0;
 }
@@ -673,6 +879,94 @@ int launch_gemv_dot4(const int8_t *A, const uint8_t *B, void *out, const float *
                        args.A, args.B, args.out, args.s, args.ws, args.M, args.N, args.K,
                        args.lpr_log2, args.passes, args.out_f32, args.div_magic, g.waves * 64);
     note_kernel("gemv_dot4_kernel", BITS, g.mt, 1 << g.batch_index, scale_kind == 1 && out_kind != OUT_G32, out_kind == OUT_G32);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+// ---- fused forms: table, set-up, launch ------------------------------------------------
+using FusedKernelFn = void (*)(const int8_t *, const uint8_t *, void *, const void *, const uint16_t *,
+                               int, int, int, int, int, int, void *);
+constexpr int kFusedMaxTile = 2;
+
+template <int BITS>
+struct FusedKernelTable {
+    FusedKernelFn fn[2][kFusedMaxTile][kBatchKinds];  // [FUSE - 1][MT - 1][batch index]
+};
+
+template <int BITS>
+const FusedKernelTable<BITS> &fused_kernel_table() {
+    static const FusedKernelTable<BITS> table = [] {
+        FusedKernelTable<BITS> t{};
+        t.fn[0][0][0] = gemv_dot4_fused_kernel<BITS, 1, 1, FUSE_SILU_PAIR>;
+        t.fn[0][0][1] = gemv_dot4_fused_kernel<BITS, 1, 2, FUSE_SILU_PAIR>;
+        t.fn[0][0][2] = gemv_dot4_fused_kernel<BITS, 1, 4, FUSE_SILU_PAIR>;
+        t.fn[0][1][0] = gemv_dot4_fused_kernel<BITS, 2, 1, FUSE_SILU_PAIR>;
+        t.fn[0][1][1] = gemv_dot4_fused_kernel<BITS, 2, 2, FUSE_SILU_PAIR>;
+        t.fn[1][0][0] = gemv_dot4_fused_kernel<BITS, 1, 1, FUSE_BF16_ACT>;
+        t.fn[1][0][1] = gemv_dot4_fused_kernel<BITS, 1, 2, FUSE_BF16_ACT>;
+        t.fn[1][0][2] = gemv_dot4_fused_kernel<BITS, 1, 4, FUSE_BF16_ACT>;
+        t.fn[1][1][0] = gemv_dot4_fused_kernel<BITS, 2, 1, FUSE_BF16_ACT>;
+        t.fn[1][1][1] = gemv_dot4_fused_kernel<BITS, 2, 2, FUSE_BF16_ACT>;
+        return t;
+    }();
+    return table;
+}
+
+template <int BITS>
+int init_fused_kernels(int max_lds) {
+    const FusedKernelTable<BITS> &t = fused_kernel_table<BITS>();
+    for (int f = 0; f < 2; ++f)
+        for (int mt = 0; mt < kFusedMaxTile; ++mt)
+            for (int u = 0; u < kBatchKinds; ++u)
+                if (t.fn[f][mt][u] != nullptr &&
+                    hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[f][mt][u]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, max_lds) != hipSuccess)
+                    return 2;
+    return 0;
+}
+
+// Geometry of a fused form; mt == 0 when the shape is not taken.
+template <int BITS>
+Geometry fused_geometry(int fuse, int M, int N, int K, int lds_limit) {
+    Geometry g = pick_geometry<BITS>(M, N, K, lds_limit - 64, lib_state<BITS>().tuning);
+    if (g.mt != 0 && fuse == FUSE_SILU_PAIR && g.lpr_log2 > 5) {
+        // the halves of a column meet in neighbouring lane sets of one wave: at most 32 lanes a row
+        Tuning tu = lib_state<BITS>().tuning;
+        tu.lanes_per_row = 32;
+        g = pick_geometry<BITS>(M, N, K, lds_limit - 64, tu);
+    }
+    if (g.mt != 0 && fuse == FUSE_SILU_PAIR && g.grid_x > kAmaxMaxParts) {
+        // few enough workgroups for the consumer to read every part with one load per lane
+        Tuning tu = lib_state<BITS>().tuning;
+        tu.lanes_per_row = 1 << g.lpr_log2;
+        tu.waves_per_wg = kMaxThreads / 64;
+        const long rows_per_pass = (long)(64 >> g.lpr_log2) * tu.waves_per_wg;
+        tu.passes = (int)((((long)N + rows_per_pass - 1) / rows_per_pass + kAmaxMaxParts - 1) / kAmaxMaxParts);
+        g = pick_geometry<BITS>(M, N, K, lds_limit - 64, tu);
+    }
+    if (g.mt > kFusedMaxTile || g.ntiles != 1 || (fuse == FUSE_SILU_PAIR && g.grid_x > kAmaxMaxParts))
+        g.mt = 0;
+    if (fuse == FUSE_SILU_PAIR) g.lds += 64;  // the waves' meeting point
+    return g;
+}
+
+// Launches a fused form for a validated shape (M <= 2) on an initialised device.  `A` is int8
+// [M, K] with multipliers `s` for FUSE_SILU_PAIR, bf16 [M, K] for FUSE_BF16_ACT.
+template <int BITS>
+int launch_gemv_dot4_fused(int fuse, const void *A, const uint8_t *B, void *out, const float *s,
+                           const void *ws, int M, int N, int K, int out_kind, uint16_t *amax,
+                           int amax_parts, float *s_out, int lds_limit, hipStream_t stream) {
+    const Geometry g = fused_geometry<BITS>(fuse, M, N, K, lds_limit);
+    if (g.mt == 0) return 1;
+    const FusedKernelFn fn = fused_kernel_table<BITS>().fn[fuse - 1][g.mt - 1][g.batch_index];
+    if (fn == nullptr) return 1;
+    const int geom = g.lpr_log2 | (g.passes << 8) | ((out_kind == OUT_F32 ? 1 : 0) << 16);
+    const bool pair = fuse == FUSE_SILU_PAIR;
+    hipLaunchKernelGGL(fn, dim3(g.grid_x, 1, 1), dim3(g.waves * 64, 1, 1), g.lds, stream,
+                       reinterpret_cast<const int8_t *>(A), B, out,
+                       pair ? static_cast<const void *>(s) : static_cast<const void *>(amax),
+                       reinterpret_cast<const uint16_t *>(ws), M, N, K, geom, pair ? g.grid_x : amax_parts,
+                       g.waves * 64, pair ? static_cast<void *>(amax) : static_cast<void *>(s_out));
+    note_kernel("gemv_dot4_fused_kernel", BITS, g.mt, 1 << g.batch_index, fuse);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

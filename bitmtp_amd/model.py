@@ -19,6 +19,7 @@ PyTorch supplies device memory, the embedding gather and graph capture only.
 from __future__ import annotations
 
 import ctypes
+import os
 import math
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
@@ -363,6 +364,10 @@ class Workspace:
         self.f_q = buf((m_max, args.dim), i8)
         self.f_s = buf((m_max,), f32)
         self.gu = buf((m_max, 2 * args.ffn_dim), bf)
+        # the MLP tail as two launches (blocks of one or two tokens): SiLU(gate) * up in bf16 and
+        # the per-workgroup maxima its quantisation needs (at most 1024 per token)
+        self.inner = buf((m_max, args.ffn_dim), bf)
+        self.inner_amax = buf((min(m_max, 2), 1024), bf)
         self.i_q = buf((m_max, args.ffn_dim), i8)
         self.i_s = buf((m_max,), f32)
         self.ffn_out = buf((m_max, args.dim), bf)
@@ -443,6 +448,39 @@ def _gemv(a_q: torch.Tensor, a_s: torch.Tensor, w: PackedLinear, out: torch.Tens
         raise RuntimeError(f"{'t2g128' if w.bits == 2 else 'q1g128'}_gemv_ex failed with status {rc}")
 
 
+def _mlp_tail_fused(lw, ws: Workspace, m: int, parts: int, stream: ctypes.c_void_p) -> None:
+    """gate|up projection with SiLU(gate) * up in its epilogue, then the down projection that
+    quantises that product while staging it: the two launches that stand for projection,
+    SiLU * up + quantisation (reference: model.py:1059-1061) and projection.  Same bits."""
+    t2 = lw.w_gu.bits == 2
+    lib = ops.t2_lib() if t2 else ops.q1_lib()
+    pair = lib.t2g128_gemv_silu_pair if t2 else lib.q1g128_gemv_silu_pair
+    act = lib.t2g128_gemv_bf16_act if t2 else lib.q1g128_gemv_bf16_act
+    rc = pair(_vp(ws.f_q), _vp(lw.w_gu.weight), _vp(ws.inner), _vp(ws.f_s), _vp(lw.w_gu.weight_scale),
+              m, lw.w_gu.out_features, lw.w_gu.in_features, _vp(ws.inner_amax), stream)
+    if rc != 0:
+        raise RuntimeError(f"gemv_silu_pair failed with status {rc}")
+    rc = act(_vp(ws.inner), _vp(lw.w_down.weight), _vp(ws.ffn_out), _vp(lw.w_down.weight_scale), m,
+             lw.w_down.out_features, lw.w_down.in_features, _vp(ws.inner_amax), parts, None,
+             ops.OUT_BF16, stream)
+    if rc != 0:
+        raise RuntimeError(f"gemv_bf16_act failed with status {rc}")
+
+
+def mlp_tail_parts(model: "BonsaiDecoder", m: int) -> int:
+    """Parts per token of the fused MLP tail at block width ``m``, 0 when the three-launch form
+    runs (wider blocks, fp16 scales, shapes the fused kernels do not take, BONSAI_FUSED_MLP=0)."""
+    if m > 2 or os.environ.get("BONSAI_FUSED_MLP", "1") == "0":
+        return 0
+    lw = model.layers[0]
+    if lw.w_gu.bits != lw.w_down.bits or lw.w_gu.weight_scale.dtype != torch.bfloat16:
+        return 0
+    lib = ops.t2_lib() if lw.w_gu.bits == 2 else ops.q1_lib()
+    fn = lib.t2g128_silu_pair_parts if lw.w_gu.bits == 2 else lib.q1g128_silu_pair_parts
+    parts = fn(m, lw.w_gu.out_features, lw.w_gu.in_features)
+    return parts if 0 < parts <= 1024 else 0
+
+
 def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tensor, sigma: int,
                  rope: Tuple[torch.Tensor, torch.Tensor], logits_start: int, logits_end: int,
                  threshold: float, head_mode: str = "native") -> None:
@@ -467,6 +505,7 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
         if rc != 0:
             raise RuntimeError(f"{what} failed with status {rc}")
 
+    tail_parts = mlp_tail_parts(model, M)
     h_cur, h_nxt = ws.h[0][:M], ws.h[1][:M]
     torch.index_select(model.embed, 0, io.tokens, out=h_cur)
     for i, lw in enumerate(model.layers):
@@ -492,11 +531,14 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
                                                  _vp(ws.f_q), _vp(ws.f_s), M, dim, stream),
               "bonsai_add_rmsnorm_quant_int8")
         h_cur, h_nxt = h_nxt, h_cur
-        _gemv(ws.f_q, ws.f_s, lw.w_gu, ws.gu, M, stream)
-        check(actq.bonsai_silu_mul_quant_int8(_vp(ws.gu), _vp(ws.i_q), _vp(ws.i_s), M,
-                                              args.ffn_dim, stream),
-              "bonsai_silu_mul_quant_int8")
-        _gemv(ws.i_q, ws.i_s, lw.w_down, ws.ffn_out, M, stream)
+        if tail_parts:
+            _mlp_tail_fused(lw, ws, M, tail_parts, stream)
+        else:
+            _gemv(ws.f_q, ws.f_s, lw.w_gu, ws.gu, M, stream)
+            check(actq.bonsai_silu_mul_quant_int8(_vp(ws.gu), _vp(ws.i_q), _vp(ws.i_s), M,
+                                                  args.ffn_dim, stream),
+                  "bonsai_silu_mul_quant_int8")
+            _gemv(ws.i_q, ws.i_s, lw.w_down, ws.ffn_out, M, stream)
 
     rows = logits_end - logits_start
     if head_mode not in ("native", "fp8", "bf16_raw"):

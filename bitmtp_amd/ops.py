@@ -35,6 +35,11 @@ _GEMV_EX_ARGTYPES = [
     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
     ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
 ]
+# (A, B, inner, s, ws, M, N2, K, amax, stream) and
+# (inner, B, out, ws, M, N, K, amax, parts, s_out, out_kind, stream)
+_SILU_PAIR_ARGTYPES = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p] * 2
+_BF16_ACT_ARGTYPES = ([ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 +
+                      [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p])
 
 
 class GemvDesc(ctypes.Structure):
@@ -95,6 +100,12 @@ def load_t2_kernel() -> None:
     lib.t2g128_last_kernel.restype = ctypes.c_char_p
     lib.t2g128_launch_count.argtypes = []
     lib.t2g128_launch_count.restype = ctypes.c_int
+    lib.t2g128_silu_pair_parts.argtypes = [ctypes.c_int] * 3
+    lib.t2g128_silu_pair_parts.restype = ctypes.c_int
+    lib.t2g128_gemv_silu_pair.argtypes = _SILU_PAIR_ARGTYPES
+    lib.t2g128_gemv_silu_pair.restype = ctypes.c_int
+    lib.t2g128_gemv_bf16_act.argtypes = _BF16_ACT_ARGTYPES
+    lib.t2g128_gemv_bf16_act.restype = ctypes.c_int
     _t2_lib = lib
 
 
@@ -127,6 +138,12 @@ def load_q1_kernel() -> None:
     lib.q1g128_last_kernel.restype = ctypes.c_char_p
     lib.q1g128_launch_count.argtypes = []
     lib.q1g128_launch_count.restype = ctypes.c_int
+    lib.q1g128_silu_pair_parts.argtypes = [ctypes.c_int] * 3
+    lib.q1g128_silu_pair_parts.restype = ctypes.c_int
+    lib.q1g128_gemv_silu_pair.argtypes = _SILU_PAIR_ARGTYPES
+    lib.q1g128_gemv_silu_pair.restype = ctypes.c_int
+    lib.q1g128_gemv_bf16_act.argtypes = _BF16_ACT_ARGTYPES
+    lib.q1g128_gemv_bf16_act.restype = ctypes.c_int
     _q1_lib = lib
 
 
@@ -380,6 +397,100 @@ def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[tor
     with torch.cuda.device(dev):
         rc = fn(_ptr(a_int8), _ptr(b_packed), _ptr(out), _ptr(s), _ptr(ws), m, n, k, out_kind,
                 scale_kind, _stream(dev))
+    if rc != 0:
+        raise RuntimeError(f"{kind}: native launch failed with status {rc} (M={m}, N={n}, K={k})")
+    return out
+
+
+FUSED_MLP_MAX_TOKENS = 2
+
+
+def silu_pair_parts(m: int, n2: int, k: int, *, bits: int) -> int:
+    """Maxima per token that :func:`packed_gemv_silu_pair` writes for this shape (the number
+    of workgroups of its launch); 0 when the shape is not taken."""
+    fn = t2_lib().t2g128_silu_pair_parts if bits == 2 else q1_lib().q1g128_silu_pair_parts
+    parts = fn(m, n2, k)
+    if parts < -1:
+        raise RuntimeError(f"silu_pair_parts: native set-up failed with status {-parts}")
+    return max(parts, 0)
+
+
+def packed_gemv_silu_pair(a_int8: torch.Tensor, b_gate_up: torch.Tensor, s: torch.Tensor,
+                          ws: torch.Tensor, *, bits: int, inner: Optional[torch.Tensor] = None,
+                          amax: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, int]:
+    """The merged gate|up projection (rows ``[gate; up]``) of one or two quantised tokens with
+    ``inner = bf16(bf16(silu(gate)) * up)`` computed in its epilogue: returns ``(inner bf16
+    [M, F], amax bf16 [M, ld], parts)`` where ``amax[m, :parts]`` holds max ``|inner[m]|`` of
+    each workgroup of the launch.  Together with :func:`packed_gemv_bf16_act` it stands for
+    projection, SiLU * up + quantisation (reference: model.py:1059-1061) and projection, with
+    the same bits."""
+    kind = "t2g128" if bits == 2 else "q1"
+    if a_int8.dim() != 2:
+        raise ValueError(f"{kind}: expected rank-2 activation")
+    _validate_packed_inputs(a_int8, b_gate_up, s, ws, kind=kind, bits=bits,
+                            activation_dtype=torch.int8, scale_dtypes=(torch.bfloat16,))
+    m, n2, k = a_int8.shape[0], b_gate_up.shape[0], b_gate_up.shape[1] * (8 // bits)
+    if m > FUSED_MLP_MAX_TOKENS or n2 % 2:
+        raise RuntimeError(f"{kind}: the fused MLP tail takes one or two tokens and an even row count")
+    dev = a_int8.device
+    with torch.cuda.device(dev):
+        parts = silu_pair_parts(m, n2, k, bits=bits)
+        if parts == 0:
+            raise RuntimeError(f"{kind}: shape not taken by the fused MLP tail (M={m}, N={n2}, K={k})")
+        ld = (parts + 7) // 8 * 8
+        if inner is None:
+            inner = torch.empty(m, n2 // 2, dtype=torch.bfloat16, device=dev)
+        if amax is None:
+            amax = torch.empty(m, ld, dtype=torch.bfloat16, device=dev)
+        if (tuple(inner.shape) != (m, n2 // 2) or inner.dtype != torch.bfloat16 or not inner.is_contiguous()
+                or amax.dtype != torch.bfloat16 or amax.numel() < m * ld or not amax.is_contiguous()
+                or inner.device != dev or amax.device != dev):
+            raise RuntimeError(f"{kind}: inner must be bf16 [{m}, {n2 // 2}] and amax bf16 with at least "
+                               f"{m * ld} elements, contiguous, on {dev}")
+        fn = t2_lib().t2g128_gemv_silu_pair if bits == 2 else q1_lib().q1g128_gemv_silu_pair
+        rc = fn(_ptr(a_int8), _ptr(b_gate_up), _ptr(inner), _ptr(s), _ptr(ws), m, n2, k, _ptr(amax),
+                _stream(dev))
+    if rc != 0:
+        raise RuntimeError(f"{kind}: native launch failed with status {rc} (M={m}, N={n2}, K={k})")
+    return inner, amax, parts
+
+
+def packed_gemv_bf16_act(inner: torch.Tensor, b_packed: torch.Tensor, ws: torch.Tensor,
+                         amax: torch.Tensor, parts: int, *, bits: int, out_kind: int = OUT_BF16,
+                         out: Optional[torch.Tensor] = None,
+                         s_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Projection of bf16 activations ``inner [M, K]`` (one or two tokens) that are quantised
+    per token while they are staged, with ``s = fl(fl(1 / max(amax, 1e-5)) * 127)`` taken from
+    the ``parts`` maxima per token that :func:`packed_gemv_silu_pair` left in ``amax``; ``s_out``
+    (fp32 [M]) receives the multipliers when given."""
+    kind = "t2g128" if bits == 2 else "q1"
+    if inner.dim() != 2 or inner.dtype != torch.bfloat16 or not inner.is_contiguous() or not inner.is_cuda:
+        raise RuntimeError(f"{kind}: expected contiguous rank-2 bf16 CUDA activations")
+    m, n, k = inner.shape[0], b_packed.shape[0], b_packed.shape[1] * (8 // bits)
+    if inner.shape[1] != k or m > FUSED_MLP_MAX_TOKENS:
+        raise RuntimeError(f"{kind}: inner must be [M <= {FUSED_MLP_MAX_TOKENS}, {k}]")
+    if ws.dtype != torch.bfloat16 or tuple(ws.shape) != (n, k // 128):
+        raise RuntimeError(f"{kind}: weight scales must be bf16 [{n}, {k // 128}]")
+    if out_kind not in (OUT_BF16, OUT_F32):
+        raise ValueError("bad out_kind")
+    ld = (parts + 7) // 8 * 8
+    if amax.dtype != torch.bfloat16 or amax.numel() < m * ld or parts < 1 or not amax.is_contiguous():
+        raise RuntimeError(f"{kind}: amax must be contiguous bf16 with at least {m * ld} elements")
+    dev = inner.device
+    dtype = torch.bfloat16 if out_kind == OUT_BF16 else torch.float32
+    if out is None:
+        out = torch.empty(m, n, dtype=dtype, device=dev)
+    elif tuple(out.shape) != (m, n) or out.dtype != dtype or out.device != dev or not out.is_contiguous():
+        raise RuntimeError(f"{kind}: out must be a contiguous {dtype} tensor of shape {(m, n)} on {dev}")
+    if s_out is not None and (s_out.dtype != torch.float32 or s_out.numel() < m or s_out.device != dev):
+        raise RuntimeError(f"{kind}: s_out must be fp32 with at least {m} elements on {dev}")
+    for t in (b_packed, ws, amax):
+        if t.device != dev:
+            raise RuntimeError(f"{kind}: all operands must be on {dev}")
+    fn = t2_lib().t2g128_gemv_bf16_act if bits == 2 else q1_lib().q1g128_gemv_bf16_act
+    with torch.cuda.device(dev):
+        rc = fn(_ptr(inner), _ptr(b_packed), _ptr(out), _ptr(ws), m, n, k, _ptr(amax), parts,
+                _ptr(s_out), out_kind, _stream(dev))
     if rc != 0:
         raise RuntimeError(f"{kind}: native launch failed with status {rc} (M={m}, N={n}, K={k})")
     return out

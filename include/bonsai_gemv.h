@@ -115,6 +115,42 @@ int t2g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, 
 int q1g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, int scale_kind,
                         void *stream);
 
+/* ---- the MLP tail as two launches (blocks of one or two tokens) ---------------------- */
+/* No counterpart in the reference, which runs gate|up projection, a torch.compile'd helper
+ * (inner = silu(gate) * up, then `quant_input`; src/bonsai_sft/gpu/model.py:1058-1061) and
+ * the down projection as three launches.  For one or two tokens every launch of a decode step
+ * costs about as much as the projection itself, so the middle one is folded into its
+ * neighbours; the operations and their rounding points are those of the three-launch form
+ * (bonsai_silu_mul_quant_int8 between two *_gemv_ex calls with BONSAI_SCALE_BF16 on the dot4
+ * kernels) and the results are the same bits.
+ *
+ * *_gemv_silu_pair: B holds the merged rows [gate (F rows); up (F rows)], N2 = 2 F.  Computes
+ *   both projections of A (int8 [M, K], multipliers s) and writes
+ *   inner = bf16(bf16(silu(gate)) * up) as bf16 [M, F]; the bf16 rounded projections themselves
+ *   are not stored.  amax (bf16, 16-byte aligned, [M, ld] with ld = parts rounded up to a
+ *   multiple of 8) receives max |inner[m]| over the columns of each of the launch's `parts`
+ *   workgroups; every element of [M, ld] is written.  parts = *_silu_pair_parts(M, N2, K)
+ *   depends on the shape only (at most 1024).
+ * *_gemv_bf16_act: projects inner (bf16 [M, K]) after quantising it per token while staging:
+ *   s[m] = fl(fl(1 / max(max_p amax[m][p], 1e-5)) * 127), q = clamp(rne(fl(inner * s)), -128, 127),
+ *   as bonsai_act_quant_int8 would; out is bf16 or fp32 [M, N] (BONSAI_OUT_BF16 / _F32);
+ *   s_out (fp32 [M], may be NULL) receives the multipliers.
+ * M <= 2; bf16 weight scales; other operands as for *_gemv_ex.  *_silu_pair_parts returns -1
+ * for a shape these kernels do not take (the caller then uses the three-launch form), -2 / -3
+ * for the set-up failures BONSAI_ERR_LAUNCH / BONSAI_ERR_NOT_INIT. */
+int t2g128_silu_pair_parts(int M, int N2, int K);
+int q1g128_silu_pair_parts(int M, int N2, int K);
+int t2g128_gemv_silu_pair(const int8_t *A, const uint8_t *B, void *inner, const float *s,
+                          const void *ws, int M, int N2, int K, void *amax, void *stream);
+int q1g128_gemv_silu_pair(const int8_t *A, const uint8_t *B, void *inner, const float *s,
+                          const void *ws, int M, int N2, int K, void *amax, void *stream);
+int t2g128_gemv_bf16_act(const void *inner, const uint8_t *B, void *out, const void *ws, int M,
+                         int N, int K, const void *amax, int parts, float *s_out, int out_kind,
+                         void *stream);
+int q1g128_gemv_bf16_act(const void *inner, const uint8_t *B, void *out, const void *ws, int M,
+                         int N, int K, const void *amax, int parts, float *s_out, int out_kind,
+                         void *stream);
+
 /* One-time set-up for the current device (raises the kernels' dynamic-LDS
  * limit).  Called implicitly by the first launch; call it explicitly before
  * capturing a graph if the first launch would otherwise happen under capture.
