@@ -425,7 +425,7 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
                                   stream);
 }
 
-// ---- the MLP tail as two launches (blocks of one or two tokens; see packed_gemv.hip.h) ------
+// ---- fused forms for blocks of one or two tokens (see packed_gemv.hip.h) ----------------------
 constexpr int kFusedMaxWidth = kFusedMaxTile;
 
 template <int BITS>
@@ -439,51 +439,47 @@ int fused_ready(int M, int N, int K, hipStream_t stream, int *lds_limit) {
     return 0;
 }
 
-// Parts per token that launch_gemv_silu_pair writes for this shape (its workgroup count), or a
-// negative status: -1 the shape is not taken, -2 / -3 as the launch statuses 2 / 3.
+// Parts per token that a fused launch with this epilogue writes for this shape (its workgroup
+// count), or a negative status: -1 the shape is not taken, -2 / -3 as the launch statuses 2 / 3.
 template <int BITS>
-int silu_pair_parts(int M, int N2, int K) {
-    if (N2 < 2 || (N2 & 1)) return -1;
+int fused_parts(int epi, int M, int N, int K) {
+    if (epi != EPI_SILU_PAIR && epi != EPI_ADD_SUMSQ) return -1;
+    if (epi == EPI_SILU_PAIR && (N < 2 || (N & 1))) return -1;
     int lds_limit = 0;
-    const int rc = fused_ready<BITS>(M, N2, K, nullptr, &lds_limit);
+    const int rc = fused_ready<BITS>(M, N, K, nullptr, &lds_limit);
     if (rc != 0) return -rc;
-    const Geometry g = fused_geometry<BITS>(FUSE_SILU_PAIR, M, N2, K, lds_limit);
+    const Geometry g = fused_geometry<BITS>(epi, M, N, K, lds_limit);
     return g.mt == 0 ? -1 : g.grid_x;
 }
 
-// gate|up projection (rows [gate; up], N2 = 2 F of them) of int8 activations: writes
-// inner = bf16(bf16(silu(gate)) * up) as bf16 [M, F] and max |inner| per token and workgroup
-// into `amax` (bf16 [M, amax_ld(parts)], parts = silu_pair_parts(M, N2, K); every element is written).
+// Validates and launches one fused GEMV.
 template <int BITS>
-int launch_gemv_silu_pair(const int8_t *A, const uint8_t *B, void *inner, const float *s, const void *ws,
-                          int M, int N2, int K, uint16_t *amax, hipStream_t stream) {
-    if (A == nullptr || B == nullptr || inner == nullptr || s == nullptr || ws == nullptr || amax == nullptr)
-        return 1;
-    if (N2 < 2 || (N2 & 1)) return 1;
-    if (!operands_aligned(A, B, inner, s, ws, OUT_BF16) || (reinterpret_cast<uintptr_t>(amax) & 15)) return 1;
+int launch_gemv_fused(const FusedGemv &d, hipStream_t stream) {
+    const auto mis = [](const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; };
+    if (d.pro < PRO_INT8 || d.pro > PRO_BF16_NORM || d.epi < EPI_PLAIN || d.epi > EPI_ADD_SUMSQ) return 1;
+    if (d.pro == PRO_INT8 && d.epi == EPI_PLAIN) return 1;  // that is *_gemv_ex
+    if (d.act == nullptr || d.B == nullptr || d.ws == nullptr || d.out == nullptr || d.act_aux == nullptr) return 1;
+    if (mis(d.act, 16) || mis(d.B, 16) || mis(d.ws, 2)) return 1;
+    if (d.pro == PRO_INT8) {
+        if (mis(d.act_aux, 4)) return 1;
+    } else if (d.pro == PRO_BF16_AMAX) {
+        if (mis(d.act_aux, 16) || d.act_parts < 1 || d.act_parts > kAmaxMaxParts) return 1;
+    } else {
+        if (mis(d.act_aux, 8) || d.act_parts < 1 || d.act_parts > kSumsqMaxParts) return 1;
+        if (d.norm_w == nullptr || mis(d.norm_w, 16) || !(d.eps >= 0.0f)) return 1;
+    }
+    if (d.s_out != nullptr && (d.pro == PRO_INT8 || mis(d.s_out, 4))) return 1;
+    if (d.epi == EPI_PLAIN) {
+        if ((d.out_kind != OUT_BF16 && d.out_kind != OUT_F32) || mis(d.out, d.out_kind == OUT_BF16 ? 2 : 4)) return 1;
+    } else {
+        if (d.out_kind != OUT_BF16 || mis(d.out, 2) || d.out_aux == nullptr) return 1;
+        if (d.epi == EPI_SILU_PAIR && (d.N < 2 || (d.N & 1) || mis(d.out_aux, 16))) return 1;
+        if (d.epi == EPI_ADD_SUMSQ && (d.residual == nullptr || mis(d.residual, 2) || mis(d.out_aux, 8))) return 1;
+    }
     int lds_limit = 0;
-    const int rc = fused_ready<BITS>(M, N2, K, stream, &lds_limit);
+    const int rc = fused_ready<BITS>(d.M, d.N, d.K, stream, &lds_limit);
     if (rc != 0) return rc;
-    return launch_gemv_dot4_fused<BITS>(FUSE_SILU_PAIR, A, B, inner, s, ws, M, N2, K, OUT_BF16, amax, 0,
-                                        nullptr, lds_limit, stream);
-}
-
-// Down projection of `inner` (bf16 [M, K]) quantised on the fly with the multiplier derived from
-// the `parts` maxima per token in `amax`; writes the multipliers to `s_out` when that is given.
-template <int BITS>
-int launch_gemv_bf16_act(const void *inner, const uint8_t *B, void *out, const void *ws, int M, int N,
-                         int K, const uint16_t *amax, int parts, float *s_out, int out_kind,
-                         hipStream_t stream) {
-    if (inner == nullptr || B == nullptr || out == nullptr || ws == nullptr || amax == nullptr) return 1;
-    if (out_kind != OUT_BF16 && out_kind != OUT_F32) return 1;
-    if (parts < 1 || parts > kAmaxMaxParts) return 1;
-    if (!operands_aligned(inner, B, out, s_out, ws, out_kind) || (reinterpret_cast<uintptr_t>(amax) & 15))
-        return 1;
-    int lds_limit = 0;
-    const int rc = fused_ready<BITS>(M, N, K, stream, &lds_limit);
-    if (rc != 0) return rc;
-    return launch_gemv_dot4_fused<BITS>(FUSE_BF16_ACT, inner, B, out, nullptr, ws, M, N, K, out_kind,
-                                        const_cast<uint16_t *>(amax), parts, s_out, lds_limit, stream);
+    return launch_gemv_dot4_fused<BITS>(d, lds_limit, stream);
 }
 
 // Several GEMVs in one call (descriptors in host memory, read before the call returns).

@@ -92,32 +92,55 @@ struct GemvArgs {
     int passes;          // row passes per wave
     int out_f32;         // 1: store the fp32 value, 0: round to bf16
     uint32_t div_magic;  // floor(2^32 / (4*C)) + 1, for task -> token in the staging loop
-    uint16_t *amax = nullptr;       // FUSE_SILU_PAIR: receives, FUSE_BF16_ACT: holds max |inner| (bf16) per token and part
-    int amax_parts = 0;             // parts per token: the workgroup count of the FUSE_SILU_PAIR launch
-    float *s_out = nullptr;         // FUSE_BF16_ACT: receives the multipliers (may be null)
+    // fused forms only (see below)
+    const void *in_parts = nullptr;       // PRO_BF16_AMAX: bf16 maxima, PRO_BF16_NORM: fp64 sums of squares
+    int in_count = 0;                     // parts per token in in_parts
+    const uint16_t *norm_w = nullptr;     // PRO_BF16_NORM: bf16 [K]
+    float eps = 0.0f;
+    const uint16_t *residual = nullptr;   // EPI_ADD_SUMSQ: bf16 [M, N]
+    void *out_parts = nullptr;            // EPI_SILU_PAIR: bf16 maxima, EPI_ADD_SUMSQ: fp64 sums of squares
+    int out_count = 0;                    // parts per token this launch writes: its workgroup count
+    float *s_out = nullptr;               // PRO_BF16_*: receives the multipliers (may be null)
 };
 
-// ---- the MLP tail without its middle launch ------------------------------------------------
-// Between the gate|up projection and the down projection the reference runs one fused Python
-// helper (src/bonsai_sft/gpu/model.py:1059-1061): inner = bf16(bf16(silu(gate)) * up), then
-// the per-token absmax quantisation of inner.  For blocks of one or two tokens that launch
-// costs as much as either projection.  Two forms of the dot4 kernel take its place:
-//   FUSE_SILU_PAIR  the gate|up projection visits its rows in the order gate 0, up 0, gate 1,
-//                   up 1, ... so that the two results of a column meet in neighbouring lane
-//                   sets; it writes inner (bf16, [M, N/2]) and, per workgroup and token, max |inner|
-//                   of what the workgroup stored (its waves meet in LDS; plain stores, no atomics
-//                   in memory -- 1536 atomic maxima spread over 32 cache lines cost 0.9 us on a
-//                   3.5 us launch, on two lines 13 us);
-//   FUSE_BF16_ACT   the down projection reads inner and the parts, derives the multiplier
-//                   s = fl(fl(1 / max(amax, 1e-5)) * 127) and quantises each value while it stages
-//                   it: q = clamp(rne(fl(x * s)), -128, 127).
-// Same operations on the same values as the three-launch form, so the results are the same bits.
-constexpr int FUSE_NONE = 0, FUSE_SILU_PAIR = 1, FUSE_BF16_ACT = 2;
-// The parts are bf16 (max |inner| is one of the bf16 values stored): up to 1024 of them are two
-// 16-byte loads per lane of a wave.
+// ---- decode steps of one or two tokens without their element-wise launches -----------------
+// Between two projections the reference runs a fused Python helper: residual add + RMSNorm +
+// quantisation (src/bonsai_sft/gpu/model.py:307-336) or SiLU(gate) * up + quantisation
+// (model.py:1059-1061).  For blocks of one or two tokens such a launch costs as much as a
+// projection.  What keeps it from being folded into its neighbours is that the quantisation (and
+// the norm) needs a value of the whole row -- max |x|, sum x^2 -- before the first element can be
+// used.  The fused forms of the dot4 kernel split that: the projection that PRODUCES a row leaves,
+// per workgroup and token, the maximum or the sum over the columns it stored (plain stores, one
+// part per workgroup: its waves meet in LDS behind a barrier at the end); the projection that
+// CONSUMES the row has every wave add up the parts (a few hundred values) and then derives the
+// multiplier and quantises while it stages.
+//   epilogues  EPI_SILU_PAIR   rows [gate; up] visited as gate 0, up 0, gate 1, up 1, ... so that the
+//                              two results of a column meet in neighbouring lane sets; stores
+//                              inner = bf16(bf16(silu(gate)) * up) [M, N/2] and max |inner| parts
+//              EPI_ADD_SUMSQ   stores h = bf16(residual + bf16(y)) [M, N] and parts of sum h^2
+//                              (fp64 sums of exact fp32 squares, in a fixed order)
+//   prologues  PRO_BF16_AMAX   x = bf16 [M, K] with max |x| parts: s = fl(fl(1 / max(amax, 1e-5)) * 127),
+//                              q = clamp(rne(fl(x * s)), -128, 127)
+//              PRO_BF16_NORM   h = bf16 [M, K] with sum h^2 parts and norm weights w:
+//                              var = fp32(sum) / K, rs = 1 / sqrt(var + eps), x = bf16(w * bf16(h * rs)),
+//                              max |x| over the workgroup (one more barrier), then as PRO_BF16_AMAX
+// The operations and their rounding points are those of the stand-alone producers (act_quant.hip),
+// so q, s and the results are the same bits as the separate launches give; the one difference is
+// the order in which the fp64 sum of squares is added up, which shows only where two fp64 roundings
+// differ and the fp32 conversion of the sum lands on the other side of a rounding boundary.
+// (Atomic maxima in memory instead of parts: 1536 of them over 32 cache lines cost 0.9 us on a
+// 3.5 us launch, over two lines 13 us.)
+constexpr int PRO_INT8 = 0, PRO_BF16_AMAX = 1, PRO_BF16_NORM = 2;
+constexpr int EPI_PLAIN = 0, EPI_SILU_PAIR = 1, EPI_ADD_SUMSQ = 2;
+constexpr int fuse_code(int pro, int epi) { return pro | (epi << 2); }
+constexpr int FUSE_NONE = 0;
+// Maxima are bf16 (max |x| is one of the bf16 values stored): up to 1024 of them are two 16-byte
+// loads per lane of a wave; sums are fp64: up to 256 of them are four 8-byte loads per lane.
 constexpr int kAmaxMaxParts = 1024;
-// elements per token of the parts array: parts rounded up to whole 16-byte words (the pad holds 0)
+constexpr int kSumsqMaxParts = 256;
+// elements per token of the maxima array: parts rounded up to whole 16-byte words (the pad holds 0)
 __host__ __device__ constexpr int amax_ld(int parts) { return (parts + 7) & ~7; }
+constexpr int kFusedMeetBytes = 64 + 2 * (kMaxThreads / 64) * 8;  // LDS behind the staged activations
 
 __device__ __forceinline__ float bf16_round_f32(float f) {
     const __bf16 b = static_cast<__bf16>(f);  // round to nearest even (v_cvt_pk_bf16_f32)
@@ -146,6 +169,32 @@ __device__ __forceinline__ u32x4 quant16_bf16(const u32x4 lo, const u32x4 hi, fl
                (q1(d1 & 0xffff0000u) << 24);
     };
     return u32x4{q4(lo.x, lo.y), q4(lo.z, lo.w), q4(hi.x, hi.y), q4(hi.z, hi.w)};
+}
+
+// Sixteen fp32 values -> sixteen int8 in natural order.
+__device__ __forceinline__ u32x4 quant16_f32(const float *v, float s) {
+    const auto q1 = [s](float x) {
+        float r = __builtin_rintf(x * s);
+        r = fminf(fmaxf(r, -128.0f), 127.0f);
+        return (uint32_t)((int)r) & 0xffu;
+    };
+    const auto q4 = [&q1](const float *x) { return q1(x[0]) | (q1(x[1]) << 8) | (q1(x[2]) << 16) | (q1(x[3]) << 24); };
+    return u32x4{q4(v), q4(v + 4), q4(v + 8), q4(v + 12)};
+}
+
+// Eight bf16 values h and their norm weights w (one 16-byte word each) -> bf16(w * bf16(h * rs)),
+// as rmsnorm_quant_kernel (act_quant.hip) evaluates it; returns max |.| of the eight.
+__device__ __forceinline__ float normalise8(const u32x4 h, const u32x4 w, float rs, float *out) {
+    const uint32_t hd[4] = {h.x, h.y, h.z, h.w}, wd[4] = {w.x, w.y, w.z, w.w};
+    float top = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[2 * i] = bf16_round_f32(__uint_as_float(wd[i] << 16) * bf16_round_f32(__uint_as_float(hd[i] << 16) * rs));
+        out[2 * i + 1] = bf16_round_f32(__uint_as_float(wd[i] & 0xffff0000u) *
+                                        bf16_round_f32(__uint_as_float(hd[i] & 0xffff0000u) * rs));
+        top = fmaxf(top, fmaxf(fabsf(out[2 * i]), fabsf(out[2 * i + 1])));
+    }
+    return top;
 }
 
 template <bool SF16>
@@ -265,6 +314,8 @@ template <int BITS, int MT, int U, bool G32, bool SF16, int FUSE = FUSE_NONE>
 __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by, int pthreads,
                                                unsigned char *smem) {
     using F = Fmt<BITS>;
+    constexpr int PRO = FUSE & 3, EPI = FUSE >> 2;
+    constexpr bool BF16_IN = PRO != PRO_INT8;
     static_assert(FUSE == FUSE_NONE || (!G32 && MT <= 2), "fused forms: one or two tokens, scaled output");
     // 4-bit planes and v_dot8 for T2 tiles of one or two tokens (see above)
     constexpr bool P4 = BITS == 2 && MT <= kPlaneMaxTile;
@@ -294,10 +345,10 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
 
     // All loads of a batch are unconditional (indices clamped into the row) and
     // issued back to back; lanes past the end of a row are masked when used.
-    // FUSE_SILU_PAIR: visiting order gate 0, up 0, gate 1, up 1, ... over the rows [gate; up]
+    // EPI_SILU_PAIR: visiting order gate 0, up 0, gate 1, up 1, ... over the rows [gate; up]
     const int half_n = N >> 1;
     auto stored_row = [&](int row) {
-        return FUSE == FUSE_SILU_PAIR ? (row & 1) * half_n + (row >> 1) : row;
+        return EPI == EPI_SILU_PAIR ? (row & 1) * half_n + (row >> 1) : row;
     };
     auto load_batch = [&](WeightBatch<U> &wb, int row, int it0) {
         const int row_c = stored_row(row < N ? row : N - 1);
@@ -316,8 +367,9 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
     // staging data (an L2 hit) is back before the weights (HBM) are.
     const int ntasks = MT * C * 4;  // quarter chunks to stage
     constexpr int kQ = F::kUnits / 4;  // 16-byte words per quarter
-    // (FUSE_BF16_ACT: a.A holds bf16 values, twice the bytes per quarter)
-    constexpr int kSrcWords = FUSE == FUSE_BF16_ACT ? 2 * kQ : kQ;
+    // (bf16 activations: twice the bytes per quarter)
+    constexpr int kSrcWords = BF16_IN ? 2 * kQ : kQ;
+    constexpr int kW = kMaxThreads / 64;
     auto task_src = [&](int task, int &m, int &chunk, int &sub) {
         if constexpr (FUSE != FUSE_NONE)
             m = (MT > 1 && task >= 4 * C) ? 1 : 0;  // at most two tokens: no division
@@ -327,37 +379,81 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
         chunk = rest >> 2;
         sub = rest & 3;
         const int msrc = (m0 + m) < M ? (m0 + m) : M - 1;
-        return reinterpret_cast<const u32x4 *>(a.A + (size_t)msrc * K * (FUSE == FUSE_BF16_ACT ? 2 : 1)) +
+        return reinterpret_cast<const u32x4 *>(a.A + (size_t)msrc * K * (BF16_IN ? 2 : 1)) +
                ((size_t)chunk * 4 + sub) * kSrcWords;
     };
+    // PRO_BF16_NORM: the norm weights of the same elements
+    auto task_w = [&](int chunk, int sub) {
+        return reinterpret_cast<const u32x4 *>(a.norm_w) + ((size_t)chunk * 4 + sub) * kSrcWords;
+    };
     u32x4 first_q[kSrcWords];
+    u32x4 first_w[PRO == PRO_BF16_NORM ? kSrcWords : 1];
     int fm = 0, fchunk = 0, fsub = 0;
     const bool has_first = tid < ntasks;
     if (has_first) {
         const u32x4 *src = task_src(tid, fm, fchunk, fsub);
 #pragma unroll
         for (int i = 0; i < kSrcWords; ++i) first_q[i] = src[i];
+        if constexpr (PRO == PRO_BF16_NORM) {
+            const u32x4 *wsrc = task_w(fchunk, fsub);
+#pragma unroll
+            for (int i = 0; i < kSrcWords; ++i) first_w[i] = wsrc[i];
+        }
     }
-    // FUSE_BF16_ACT: every wave reads the parts of a token itself, one 16-byte word per lane (a
-    // second workgroup barrier ahead of the staging costs more than the repeated reads)
+    // Every wave reads the parts of a token itself (a workgroup barrier for them costs more than
+    // the repeated reads): maxima as one or two 16-byte words per lane, sums as up to four doubles
+    // per lane, added in that order
+    // (nothing below may wait for these loads before the weight loads are issued)
     u32x4 part_bits[MT][2];
-    if (FUSE == FUSE_BF16_ACT) {
-        const int words = amax_ld(a.amax_parts) >> 3;  // at most 128
+    double part_raw[MT][4];
+    if (PRO == PRO_BF16_AMAX) {
+        const int words = amax_ld(a.in_count) >> 3;  // at most 128
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             const u32x4 *prow = reinterpret_cast<const u32x4 *>(
-                a.amax + (size_t)((m0 + m) < M ? (m0 + m) : M - 1) * (words * 8));
+                static_cast<const uint16_t *>(a.in_parts) + (size_t)((m0 + m) < M ? (m0 + m) : M - 1) * (words * 8));
             part_bits[m][0] = prow[lane < words ? lane : words - 1];  // past the end: a repeat
             part_bits[m][1] = prow[lane + 64 < words ? lane + 64 : words - 1];
+        }
+    }
+    if (PRO == PRO_BF16_NORM) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const double *prow = static_cast<const double *>(a.in_parts) +
+                                 (size_t)((m0 + m) < M ? (m0 + m) : M - 1) * a.in_count;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int idx = lane + 64 * j;
+                part_raw[m][j] = prow[idx < a.in_count ? idx : 0];  // past the end: not added below
+            }
         }
     }
 
     WeightBatch<U> cur, nxt;
     load_batch(cur, row0, 0);
-    if (FUSE == FUSE_SILU_PAIR) asm volatile("" ::"s"(a.amax));  // fetched now, used at the very end
+    // (arguments that only the end of the kernel needs are fetched now)
+    if (EPI != EPI_PLAIN) asm volatile("" ::"s"(a.out_parts), "s"(a.out_count));
+    // EPI_ADD_SUMSQ: the residual values of the first pass travel with the weights
+    // (raw, from a clamped address and untouched until the epilogue: an operation on it here would
+    // wait for the weight loads issued before it)
+    uint16_t res0[MT];
+    if constexpr (EPI == EPI_ADD_SUMSQ) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            res0[m] = a.residual[(size_t)((m0 + m) < M ? (m0 + m) : M - 1) * N + (row0 < N ? row0 : N - 1)];
+    }
 
+    // the multiplier of a token picked by a run-time index (at most two tokens)
+    auto of_token = [](const float *v, int m) {
+        float x = v[0];
+#pragma unroll
+        for (int t = 1; t < MT; ++t) x = (m == t) ? v[t] : x;
+        return x;
+    };
     float sdiv[MT];
-    if (FUSE == FUSE_BF16_ACT) {
+    float rs[MT];                                             // PRO_BF16_NORM: 1 / sqrt(var + eps)
+    float first_n[PRO == PRO_BF16_NORM ? kSrcWords * 8 : 1];  // the first task's normalised values
+    if constexpr (PRO == PRO_BF16_AMAX) {
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             // non-negative bf16 values order as unsigned 16-bit integers
@@ -374,21 +470,65 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
             const float recip = 1.0f / fmaxf(amax, 1e-5f);  // IEEE division, rounded on its own
             sdiv[m] = recip * 127.0f;
         }
-        if (bx == 0 && wave == 0) {
+    } else if constexpr (PRO == PRO_BF16_NORM) {
+        float lmax[MT];
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                if ((m0 + m) < M && a.s_out != nullptr && lane == 0) a.s_out[m0 + m] = sdiv[m];
-            }
+        for (int m = 0; m < MT; ++m) {
+            double mine = part_raw[m][0];
+            mine = lane < a.in_count ? mine : 0.0;
+#pragma unroll
+            for (int j = 1; j < 4; ++j) mine += (lane + 64 * j) < a.in_count ? part_raw[m][j] : 0.0;
+            const double total = bonsai_wave::sum64(mine);
+            const float var = (float)total / (float)K;
+            rs[m] = 1.0f / sqrtf(var + a.eps);
+            lmax[m] = 0.0f;
+        }
+        // first pass over this thread's quarters: normalise, maxima per token
+        if (has_first) {
+            float top = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kSrcWords; ++i)
+                top = fmaxf(top, normalise8(first_q[i], first_w[i], of_token(rs, fm), first_n + 8 * i));
+#pragma unroll
+            for (int m = 0; m < MT; ++m) lmax[m] = (m == fm) ? top : lmax[m];
+        }
+        for (int task = tid + nthreads; task < ntasks; task += nthreads) {
+            int m, chunk, sub;
+            const u32x4 *src = task_src(task, m, chunk, sub);
+            const u32x4 *wsrc = task_w(chunk, sub);
+            float tmp[8], top = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kSrcWords; ++i) top = fmaxf(top, normalise8(src[i], wsrc[i], of_token(rs, m), tmp));
+#pragma unroll
+            for (int t = 0; t < MT; ++t) lmax[t] = (t == m) ? fmaxf(lmax[t], top) : lmax[t];
+        }
+        float *pro_meet = reinterpret_cast<float *>(smem + (size_t)C * block_words<BITS, MT>() * 16);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float wm = bonsai_wave::max64(lmax[m]);
+            if (lane == 0) pro_meet[m * kW + wave] = wm;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            float amax = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kW; ++w) amax = fmaxf(amax, pro_meet[m * kW + (w < nwaves ? w : nwaves - 1)]);
+            const float recip = 1.0f / fmaxf(amax, 1e-5f);
+            sdiv[m] = recip * 127.0f;
         }
     } else if (!G32) {
 #pragma unroll
         for (int m = 0; m < MT; ++m) sdiv[m] = a.s[(m0 + m) < M ? (m0 + m) : M - 1];
     }
-    // FUSE_BF16_ACT: the quarter as int8, quantised with its token's multiplier
-    auto quantised = [&](const u32x4 *raw, int m, u32x4 *q) {
-        float sm = sdiv[0];
+    if (BF16_IN && bx == 0 && tid == 0 && a.s_out != nullptr) {
 #pragma unroll
-        for (int t = 1; t < MT; ++t) sm = (m == t) ? sdiv[t] : sm;
+        for (int m = 0; m < MT; ++m)
+            if ((m0 + m) < M) a.s_out[m0 + m] = sdiv[m];
+    }
+    // bf16 activations: a quarter as int8, quantised with its token's multiplier
+    auto quantised = [&](const u32x4 *raw, int m, u32x4 *q) {
+        const float sm = of_token(sdiv, m);
 #pragma unroll
         for (int i = 0; i < kQ; ++i) q[i] = quant16_bf16(raw[2 * i], raw[2 * i + 1], sm);
     };
@@ -397,8 +537,13 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
     if (has_first) {
         u32x4 fq[kQ];
         const u32x4 *fsrc = first_q;
-        if constexpr (FUSE == FUSE_BF16_ACT) {
+        if constexpr (PRO == PRO_BF16_AMAX) {
             quantised(first_q, fm, fq);
+            fsrc = fq;
+        }
+        if constexpr (PRO == PRO_BF16_NORM) {
+#pragma unroll
+            for (int i = 0; i < kQ; ++i) fq[i] = quant16_f32(first_n + 16 * i, of_token(sdiv, fm));
             fsrc = fq;
         }
         int qs;
@@ -414,11 +559,21 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
         int m, chunk, sub;
         const u32x4 *src = task_src(task, m, chunk, sub);
         u32x4 tq[kQ];
-        if constexpr (FUSE == FUSE_BF16_ACT) {
+        if constexpr (PRO == PRO_BF16_AMAX) {
             u32x4 raw[kSrcWords];
 #pragma unroll
             for (int i = 0; i < kSrcWords; ++i) raw[i] = src[i];
             quantised(raw, m, tq);
+            src = tq;
+        }
+        if constexpr (PRO == PRO_BF16_NORM) {
+            // (second pass: the values are normalised again rather than kept)
+            const u32x4 *wsrc = task_w(chunk, sub);
+            float tmp[kSrcWords * 8];
+#pragma unroll
+            for (int i = 0; i < kSrcWords; ++i) (void)normalise8(src[i], wsrc[i], of_token(rs, m), tmp + 8 * i);
+#pragma unroll
+            for (int i = 0; i < kQ; ++i) tq[i] = quant16_f32(tmp + 16 * i, of_token(sdiv, m));
             src = tq;
         }
         int qs;
@@ -430,17 +585,18 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
         qs += dpp_i32<kDppXor2>(qs);
         if (sub == 0) asum[asum_index<BITS, MT>(m, chunk)] = qs;
     }
-    // FUSE_SILU_PAIR: where the waves of the workgroup meet at the end, behind the staged
-    // activations: MT maxima per wave
-    uint32_t *meet = reinterpret_cast<uint32_t *>(smem + (size_t)C * block_words<BITS, MT>() * 16);
+    // where the waves of the workgroup meet at the end of an epilogue that leaves parts
+    unsigned char *epi_meet = smem + (size_t)C * block_words<BITS, MT>() * 16 + 64;
     __syncthreads();
 
     float accf[MT];
-    float inner_max[MT];  // FUSE_SILU_PAIR: max |inner| this lane has stored
+    float inner_max[MT];  // EPI_SILU_PAIR: max |inner| this lane has stored
+    double sumsq[MT];     // EPI_ADD_SUMSQ: sum of the squares this lane has stored
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         accf[m] = 0.0f;
         inner_max[m] = 0.0f;
+        sumsq[m] = 0.0;
     }
 
     // One batch of one pass: unpack, dot, scale, and after the last batch of the
@@ -484,7 +640,18 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
             for (int m = 0; m < MT; ++m) {
                 const float sum = row_lanes_sum(accf[m], lpr_log2);
                 accf[m] = 0.0f;
-                if constexpr (FUSE == FUSE_SILU_PAIR) {
+                if constexpr (EPI == EPI_ADD_SUMSQ) {
+                    if (c == 0 && row_ok && (m0 + m) < M) {
+                        const size_t o = (size_t)(m0 + m) * N + row;
+                        const float res = __uint_as_float((uint32_t)(pass == 0 ? res0[m] : a.residual[o]) << 16);
+                        const float hv = bf16_round_f32(bf16_round_f32(sum / sdiv[m]) + res);
+                        reinterpret_cast<uint16_t *>(a.out)[o] = (uint16_t)(__float_as_uint(hv) >> 16);
+                        const float sq = hv * hv;  // exact: two 8-bit significands
+                        sumsq[m] += (double)sq;
+                    }
+                    continue;
+                }
+                if constexpr (EPI == EPI_SILU_PAIR) {
                     // every lane of a row's set holds the row's value; the next set (row ^ 1)
                     // holds the other half of the column
                     const float mine = bf16_round_f32(sum / sdiv[m]);
@@ -543,13 +710,13 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
     } else {
         compute_batch(cur, pa, ba);
     }
-    if constexpr (FUSE == FUSE_SILU_PAIR) {
+    if constexpr (EPI == EPI_SILU_PAIR) {
         // the waves' maxima meet in LDS behind a barrier (every wave is at its end by then) and
         // thread 0 stores the workgroup's part.  Measured on 12288 x 2048 at one token (3.45 us as
         // a plain GEMV, 3.70 us with the pairing and SiLU alone): this barrier 3.97 us, a count in
         // LDS whose last arriver stores 4.14 us, one part per wave 3.83 us (but four times the
         // parts for every wave of the consumer to read)
-        constexpr int kW = kMaxThreads / 64;
+        uint32_t *meet = reinterpret_cast<uint32_t *>(epi_meet);
         float wmax[MT];
 #pragma unroll
         for (int m = 0; m < MT; ++m) wmax[m] = bonsai_wave::max64(inner_max[m]);
@@ -559,7 +726,7 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
         }
         __syncthreads();
         if (tid == 0) {
-            const int parts = a.amax_parts, ld = amax_ld(parts);  // (the grid size, as a parameter)
+            const int parts = a.out_count, ld = amax_ld(parts);  // (the grid size, as a parameter)
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 if ((m0 + m) >= M) continue;
@@ -569,10 +736,35 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
                     const uint32_t v = meet[m * kW + (w < nwaves ? w : nwaves - 1)];
                     top = v > top ? v : top;
                 }
-                uint16_t *prow = a.amax + (size_t)(m0 + m) * ld;
+                uint16_t *prow = static_cast<uint16_t *>(a.out_parts) + (size_t)(m0 + m) * ld;
                 prow[bx] = (uint16_t)(top >> 16);  // exact: one of the bf16 values stored
                 if (bx == parts - 1)
                     for (int w = parts; w < ld; ++w) prow[w] = 0;
+            }
+        }
+    }
+    if constexpr (EPI == EPI_ADD_SUMSQ) {
+        // the same meeting for the sums: a wave's lanes on the DPP butterfly, the waves left to right
+        double *meet = reinterpret_cast<double *>(epi_meet);
+        double wsum[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) wsum[m] = bonsai_wave::sum64(sumsq[m]);
+        if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) meet[m * kW + wave] = wsum[m];
+        }
+        __syncthreads();
+        if (tid == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if ((m0 + m) >= M) continue;
+                double v[kW];  // all slots read at once (those past nwaves hold stale words: not added)
+#pragma unroll
+                for (int w = 0; w < kW; ++w) v[w] = meet[m * kW + w];
+                double t = v[0];
+#pragma unroll
+                for (int w = 1; w < kW; ++w) t += w < nwaves ? v[w] : 0.0;
+                static_cast<double *>(a.out_parts)[(size_t)(m0 + m) * a.out_count + bx] = t;
             }
         }
     }
@@ -589,28 +781,33 @@ gemv_dot4_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const float *p
     gemv_dot4_body<BITS, MT, U, G32, SF16>(a, (int)blockIdx.x, (int)blockIdx.y, pthreads, smem);
 }
 
-// The fused forms (FUSE_SILU_PAIR, FUSE_BF16_ACT) of the same body; bf16 scales, bf16 or fp32 out.
+// The fused forms of the same body; bf16 scales.
 // Sixteen dwords of arguments arrive in SGPRs with the wave; a later one is a scalar load that
-// the compiler places where the value is first needed.  So `px` is what the prologue needs (the
-// multipliers for FUSE_SILU_PAIR, the parts for FUSE_BF16_ACT) and `py` what only the end of the
-// kernel needs (the parts to write / the optional multiplier output); the body asks for `py` once
-// its first loads are on their way.  pgeom = lpr_log2 | passes << 8 | out_f32 << 16.
+// the compiler places where the value is first needed (0.3 us when that is the end of the last
+// wave of a workgroup).  So the first sixteen are what the prologue needs -- `px` the multipliers
+// (PRO_INT8) or the parts to read, `pw` the norm weights -- and the body asks for what only the
+// end of the kernel needs once its first loads are on their way.
+// pgeom = lpr_log2 | passes << 4 | out_f32 << 9 | waves << 10 | parts to read << 14.
 template <int BITS, int MT, int U, int FUSE>
 __global__ void __launch_bounds__(kMaxThreads)
-gemv_dot4_fused_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const void *px,
-                       const uint16_t *pws, int pM, int pN, int pK, int pgeom, int pparts,
-                       int pthreads, void *py) {
-    GemvArgs a{pA, pB, pout, nullptr, pws, pM, pN, pK, pgeom & 0xff, (pgeom >> 8) & 0xff, (pgeom >> 16) & 1, 0u};
-    if (FUSE == FUSE_SILU_PAIR) {
+gemv_dot4_fused_kernel(const int8_t *pA, const uint8_t *pB, void *pout, const uint16_t *pws,
+                       const void *px, const uint16_t *pw, int pM, int pN, int pK, int pgeom,
+                       float peps, void *py, const uint16_t *pr, int pout_count, float *ps_out) {
+    GemvArgs a{pA, pB, pout, nullptr, pws, pM, pN, pK, pgeom & 0xf, (pgeom >> 4) & 0x1f, (pgeom >> 9) & 1, 0u};
+    if ((FUSE & 3) == PRO_INT8)
         a.s = static_cast<const float *>(px);
-        a.amax = static_cast<uint16_t *>(py);
-    } else {
-        a.amax = const_cast<uint16_t *>(static_cast<const uint16_t *>(px));
-        a.s_out = static_cast<float *>(py);
-    }
-    a.amax_parts = pparts;
+    else
+        a.in_parts = px;
+    a.in_count = (pgeom >> 14) & 0x7ff;
+    a.norm_w = pw;
+    a.eps = peps;
+    a.residual = pr;
+    a.out_parts = py;
+    a.out_count = pout_count;
+    a.s_out = ps_out;
     extern __shared__ __align__(16) unsigned char smem[];
-    gemv_dot4_body<BITS, MT, U, false, false, FUSE>(a, (int)blockIdx.x, (int)blockIdx.y, pthreads, smem);
+    gemv_dot4_body<BITS, MT, U, false, false, FUSE>(a, (int)blockIdx.x, (int)blockIdx.y,
+                                                    ((pgeom >> 10) & 0xf) * 64, smem);
 }
 
 // ---- several GEMVs in one launch -------------------------------------------------------
@@ -883,29 +1080,55 @@ int launch_gemv_dot4(const int8_t *A, const uint8_t *B, void *out, const float *
 }
 
 // ---- fused forms: table, set-up, launch ------------------------------------------------
-using FusedKernelFn = void (*)(const int8_t *, const uint8_t *, void *, const void *, const uint16_t *,
-                               int, int, int, int, int, int, void *);
+using FusedKernelFn = void (*)(const int8_t *, const uint8_t *, void *, const uint16_t *, const void *,
+                               const uint16_t *, int, int, int, int, float, void *, const uint16_t *, int,
+                               float *);
 constexpr int kFusedMaxTile = 2;
+
+// One fused GEMV (host side; the C structure of the entry point carries the same fields).
+struct FusedGemv {
+    int pro, epi;
+    const void *act;      // int8 [M, K] (PRO_INT8) or bf16 [M, K]
+    const void *act_aux;  // PRO_INT8: fp32 s[M]; PRO_BF16_AMAX: bf16 maxima; PRO_BF16_NORM: fp64 sums
+    int act_parts;        // parts per token in act_aux
+    const uint16_t *norm_w;
+    float eps;
+    const uint8_t *B;
+    const void *ws;
+    void *out;            // EPI_PLAIN: bf16 / fp32 [M, N]; EPI_SILU_PAIR: bf16 [M, N/2]; EPI_ADD_SUMSQ: bf16 [M, N]
+    const uint16_t *residual;
+    void *out_aux;        // EPI_SILU_PAIR: bf16 maxima [M, amax_ld(parts)]; EPI_ADD_SUMSQ: fp64 sums [M, parts]
+    float *s_out;
+    int M, N, K, out_kind;
+};
 
 template <int BITS>
 struct FusedKernelTable {
-    FusedKernelFn fn[2][kFusedMaxTile][kBatchKinds];  // [FUSE - 1][MT - 1][batch index]
+    FusedKernelFn fn[3][3][kFusedMaxTile][kBatchKinds];  // [prologue][epilogue][MT - 1][batch index]
 };
 
+template <int BITS, int PRO, int EPI>
+void fill_fused_cells(FusedKernelTable<BITS> &t) {
+    constexpr int F = fuse_code(PRO, EPI);
+    t.fn[PRO][EPI][0][0] = gemv_dot4_fused_kernel<BITS, 1, 1, F>;
+    t.fn[PRO][EPI][0][1] = gemv_dot4_fused_kernel<BITS, 1, 2, F>;
+    t.fn[PRO][EPI][0][2] = gemv_dot4_fused_kernel<BITS, 1, 4, F>;
+    t.fn[PRO][EPI][1][0] = gemv_dot4_fused_kernel<BITS, 2, 1, F>;
+    t.fn[PRO][EPI][1][1] = gemv_dot4_fused_kernel<BITS, 2, 2, F>;
+}
+
+// The combinations a decode layer uses (q|k|v: norm in; o: residual out; gate|up: norm in, SiLU
+// pair out; down: maxima in, residual out) and the two of the MLP tail on its own.
 template <int BITS>
 const FusedKernelTable<BITS> &fused_kernel_table() {
     static const FusedKernelTable<BITS> table = [] {
         FusedKernelTable<BITS> t{};
-        t.fn[0][0][0] = gemv_dot4_fused_kernel<BITS, 1, 1, FUSE_SILU_PAIR>;
-        t.fn[0][0][1] = gemv_dot4_fused_kernel<BITS, 1, 2, FUSE_SILU_PAIR>;
-        t.fn[0][0][2] = gemv_dot4_fused_kernel<BITS, 1, 4, FUSE_SILU_PAIR>;
-        t.fn[0][1][0] = gemv_dot4_fused_kernel<BITS, 2, 1, FUSE_SILU_PAIR>;
-        t.fn[0][1][1] = gemv_dot4_fused_kernel<BITS, 2, 2, FUSE_SILU_PAIR>;
-        t.fn[1][0][0] = gemv_dot4_fused_kernel<BITS, 1, 1, FUSE_BF16_ACT>;
-        t.fn[1][0][1] = gemv_dot4_fused_kernel<BITS, 1, 2, FUSE_BF16_ACT>;
-        t.fn[1][0][2] = gemv_dot4_fused_kernel<BITS, 1, 4, FUSE_BF16_ACT>;
-        t.fn[1][1][0] = gemv_dot4_fused_kernel<BITS, 2, 1, FUSE_BF16_ACT>;
-        t.fn[1][1][1] = gemv_dot4_fused_kernel<BITS, 2, 2, FUSE_BF16_ACT>;
+        fill_fused_cells<BITS, PRO_INT8, EPI_SILU_PAIR>(t);
+        fill_fused_cells<BITS, PRO_INT8, EPI_ADD_SUMSQ>(t);
+        fill_fused_cells<BITS, PRO_BF16_AMAX, EPI_PLAIN>(t);
+        fill_fused_cells<BITS, PRO_BF16_AMAX, EPI_ADD_SUMSQ>(t);
+        fill_fused_cells<BITS, PRO_BF16_NORM, EPI_PLAIN>(t);
+        fill_fused_cells<BITS, PRO_BF16_NORM, EPI_SILU_PAIR>(t);
         return t;
     }();
     return table;
@@ -914,59 +1137,57 @@ const FusedKernelTable<BITS> &fused_kernel_table() {
 template <int BITS>
 int init_fused_kernels(int max_lds) {
     const FusedKernelTable<BITS> &t = fused_kernel_table<BITS>();
-    for (int f = 0; f < 2; ++f)
-        for (int mt = 0; mt < kFusedMaxTile; ++mt)
-            for (int u = 0; u < kBatchKinds; ++u)
-                if (t.fn[f][mt][u] != nullptr &&
-                    hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[f][mt][u]),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, max_lds) != hipSuccess)
-                    return 2;
+    for (int p = 0; p < 3; ++p)
+        for (int e = 0; e < 3; ++e)
+            for (int mt = 0; mt < kFusedMaxTile; ++mt)
+                for (int u = 0; u < kBatchKinds; ++u)
+                    if (t.fn[p][e][mt][u] != nullptr &&
+                        hipFuncSetAttribute(reinterpret_cast<const void *>(t.fn[p][e][mt][u]),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, max_lds) != hipSuccess)
+                        return 2;
     return 0;
 }
 
-// Geometry of a fused form; mt == 0 when the shape is not taken.
+// Geometry of a fused form (it depends on the epilogue only); mt == 0 when the shape is not taken.
 template <int BITS>
-Geometry fused_geometry(int fuse, int M, int N, int K, int lds_limit) {
-    Geometry g = pick_geometry<BITS>(M, N, K, lds_limit - 64, lib_state<BITS>().tuning);
-    if (g.mt != 0 && fuse == FUSE_SILU_PAIR && g.lpr_log2 > 5) {
+Geometry fused_geometry(int epi, int M, int N, int K, int lds_limit) {
+    const int lds_left = lds_limit - kFusedMeetBytes;
+    Geometry g = pick_geometry<BITS>(M, N, K, lds_left, lib_state<BITS>().tuning);
+    if (g.mt != 0 && epi == EPI_SILU_PAIR && g.lpr_log2 > 5) {
         // the halves of a column meet in neighbouring lane sets of one wave: at most 32 lanes a row
         Tuning tu = lib_state<BITS>().tuning;
         tu.lanes_per_row = 32;
-        g = pick_geometry<BITS>(M, N, K, lds_limit - 64, tu);
+        g = pick_geometry<BITS>(M, N, K, lds_left, tu);
     }
-    if (g.mt != 0 && fuse == FUSE_SILU_PAIR && g.grid_x > kAmaxMaxParts) {
-        // few enough workgroups for the consumer to read every part with one load per lane
+    const int max_parts = epi == EPI_SILU_PAIR ? kAmaxMaxParts : (epi == EPI_ADD_SUMSQ ? kSumsqMaxParts : 1 << 30);
+    if (g.mt != 0 && g.grid_x > max_parts) {
+        // few enough workgroups for the consumer's waves to read every part with a few loads
         Tuning tu = lib_state<BITS>().tuning;
         tu.lanes_per_row = 1 << g.lpr_log2;
         tu.waves_per_wg = kMaxThreads / 64;
         const long rows_per_pass = (long)(64 >> g.lpr_log2) * tu.waves_per_wg;
-        tu.passes = (int)((((long)N + rows_per_pass - 1) / rows_per_pass + kAmaxMaxParts - 1) / kAmaxMaxParts);
-        g = pick_geometry<BITS>(M, N, K, lds_limit - 64, tu);
+        tu.passes = (int)((((long)N + rows_per_pass - 1) / rows_per_pass + max_parts - 1) / max_parts);
+        g = pick_geometry<BITS>(M, N, K, lds_left, tu);
     }
-    if (g.mt > kFusedMaxTile || g.ntiles != 1 || (fuse == FUSE_SILU_PAIR && g.grid_x > kAmaxMaxParts))
-        g.mt = 0;
-    if (fuse == FUSE_SILU_PAIR) g.lds += 64;  // the waves' meeting point
+    if (g.mt > kFusedMaxTile || g.ntiles != 1 || g.grid_x > max_parts || g.passes > 31) g.mt = 0;
+    g.lds += kFusedMeetBytes;
     return g;
 }
 
-// Launches a fused form for a validated shape (M <= 2) on an initialised device.  `A` is int8
-// [M, K] with multipliers `s` for FUSE_SILU_PAIR, bf16 [M, K] for FUSE_BF16_ACT.
+// Launches a fused form for validated operands (M <= 2) on an initialised device.
 template <int BITS>
-int launch_gemv_dot4_fused(int fuse, const void *A, const uint8_t *B, void *out, const float *s,
-                           const void *ws, int M, int N, int K, int out_kind, uint16_t *amax,
-                           int amax_parts, float *s_out, int lds_limit, hipStream_t stream) {
-    const Geometry g = fused_geometry<BITS>(fuse, M, N, K, lds_limit);
+int launch_gemv_dot4_fused(const FusedGemv &d, int lds_limit, hipStream_t stream) {
+    const Geometry g = fused_geometry<BITS>(d.epi, d.M, d.N, d.K, lds_limit);
     if (g.mt == 0) return 1;
-    const FusedKernelFn fn = fused_kernel_table<BITS>().fn[fuse - 1][g.mt - 1][g.batch_index];
+    const FusedKernelFn fn = fused_kernel_table<BITS>().fn[d.pro][d.epi][g.mt - 1][g.batch_index];
     if (fn == nullptr) return 1;
-    const int geom = g.lpr_log2 | (g.passes << 8) | ((out_kind == OUT_F32 ? 1 : 0) << 16);
-    const bool pair = fuse == FUSE_SILU_PAIR;
+    const int geom = g.lpr_log2 | (g.passes << 4) | ((d.out_kind == OUT_F32 ? 1 : 0) << 9) | (g.waves << 10) |
+                     (d.act_parts << 14);
     hipLaunchKernelGGL(fn, dim3(g.grid_x, 1, 1), dim3(g.waves * 64, 1, 1), g.lds, stream,
-                       reinterpret_cast<const int8_t *>(A), B, out,
-                       pair ? static_cast<const void *>(s) : static_cast<const void *>(amax),
-                       reinterpret_cast<const uint16_t *>(ws), M, N, K, geom, pair ? g.grid_x : amax_parts,
-                       g.waves * 64, pair ? static_cast<void *>(amax) : static_cast<void *>(s_out));
-    note_kernel("gemv_dot4_fused_kernel", BITS, g.mt, 1 << g.batch_index, fuse);
+                       reinterpret_cast<const int8_t *>(d.act), d.B, d.out,
+                       reinterpret_cast<const uint16_t *>(d.ws), d.act_aux, d.norm_w, d.M, d.N, d.K, geom,
+                       d.eps, d.out_aux, d.residual, g.grid_x, d.s_out);
+    note_kernel("gemv_dot4_fused_kernel", BITS, g.mt, 1 << g.batch_index, fuse_code(d.pro, d.epi));
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

@@ -138,18 +138,18 @@ void q1g128_int8xint1_linear(int8_t *A, int8_t *B, void *C, float *s, void *ws, 
         fprintf(stderr, "[q1g128] unsupported shape M=%d N=%d K=%d (status %d)\n", M, N, K, rc);
 }
 
-int q1g128_silu_pair_parts(int M, int N2, int K) { return silu_pair_parts<1>(M, N2, K); }
-
-int q1g128_gemv_silu_pair(const int8_t *A, const uint8_t *B, void *inner, const float *s, const void *ws,
-                          int M, int N2, int K, void *amax, void *stream) {
-    return launch_gemv_silu_pair<1>(A, B, inner, s, ws, M, N2, K, static_cast<uint16_t *>(amax),
-                                    static_cast<hipStream_t>(stream));
+static FusedGemv fused_from(const bonsai_fused_gemv *d) {
+    return FusedGemv{d->act_kind, d->epi_kind, d->act, d->act_aux, d->act_parts,
+                     static_cast<const uint16_t *>(d->norm_weight), d->eps, d->B, d->ws, d->out,
+                     static_cast<const uint16_t *>(d->residual), d->out_aux, d->s_out, d->M, d->N, d->K,
+                     d->out_kind};
 }
 
-int q1g128_gemv_bf16_act(const void *inner, const uint8_t *B, void *out, const void *ws, int M, int N, int K,
-                         const void *amax, int parts, float *s_out, int out_kind, void *stream) {
-    return launch_gemv_bf16_act<1>(inner, B, out, ws, M, N, K, static_cast<const uint16_t *>(amax), parts, s_out, out_kind,
-                                      static_cast<hipStream_t>(stream));
+int q1g128_fused_parts(int epi_kind, int M, int N, int K) { return fused_parts<1>(epi_kind, M, N, K); }
+
+int q1g128_gemv_fused(const bonsai_fused_gemv *d, void *stream) {
+    if (d == nullptr) return BONSAI_ERR_ARG;
+    return launch_gemv_fused<1>(fused_from(d), static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

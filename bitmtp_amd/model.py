@@ -364,10 +364,12 @@ class Workspace:
         self.f_q = buf((m_max, args.dim), i8)
         self.f_s = buf((m_max,), f32)
         self.gu = buf((m_max, 2 * args.ffn_dim), bf)
-        # the MLP tail as two launches (blocks of one or two tokens): SiLU(gate) * up in bf16 and
-        # the per-workgroup maxima its quantisation needs (at most 1024 per token)
+        # fused layers (blocks of one or two tokens): SiLU(gate) * up in bf16, the per-workgroup
+        # maxima its quantisation needs (at most 1024 per token) and the per-workgroup sums of
+        # squares of the residual stream (at most 256 per token)
         self.inner = buf((m_max, args.ffn_dim), bf)
         self.inner_amax = buf((min(m_max, 2), 1024), bf)
+        self.sumsq = buf((min(m_max, 2), 256), torch.float64)
         self.i_q = buf((m_max, args.ffn_dim), i8)
         self.i_s = buf((m_max,), f32)
         self.ffn_out = buf((m_max, args.dim), bf)
@@ -448,37 +450,50 @@ def _gemv(a_q: torch.Tensor, a_s: torch.Tensor, w: PackedLinear, out: torch.Tens
         raise RuntimeError(f"{'t2g128' if w.bits == 2 else 'q1g128'}_gemv_ex failed with status {rc}")
 
 
-def _mlp_tail_fused(lw, ws: Workspace, m: int, parts: int, stream: ctypes.c_void_p) -> None:
-    """gate|up projection with SiLU(gate) * up in its epilogue, then the down projection that
-    quantises that product while staging it: the two launches that stand for projection,
-    SiLU * up + quantisation (reference: model.py:1059-1061) and projection.  Same bits."""
-    t2 = lw.w_gu.bits == 2
-    lib = ops.t2_lib() if t2 else ops.q1_lib()
-    pair = lib.t2g128_gemv_silu_pair if t2 else lib.q1g128_gemv_silu_pair
-    act = lib.t2g128_gemv_bf16_act if t2 else lib.q1g128_gemv_bf16_act
-    rc = pair(_vp(ws.f_q), _vp(lw.w_gu.weight), _vp(ws.inner), _vp(ws.f_s), _vp(lw.w_gu.weight_scale),
-              m, lw.w_gu.out_features, lw.w_gu.in_features, _vp(ws.inner_amax), stream)
-    if rc != 0:
-        raise RuntimeError(f"gemv_silu_pair failed with status {rc}")
-    rc = act(_vp(ws.inner), _vp(lw.w_down.weight), _vp(ws.ffn_out), _vp(lw.w_down.weight_scale), m,
-             lw.w_down.out_features, lw.w_down.in_features, _vp(ws.inner_amax), parts, None,
-             ops.OUT_BF16, stream)
-    if rc != 0:
-        raise RuntimeError(f"gemv_bf16_act failed with status {rc}")
+@dataclass
+class FusedPlan:
+    """Parts per token that the three part-writing launches of a fused layer leave
+    (``*_fused_parts`` of include/bonsai_gemv.h)."""
+    o: int      # o projection: sums of squares
+    gu: int     # gate|up projection: maxima
+    down: int   # down projection: sums of squares
 
 
-def mlp_tail_parts(model: "BonsaiDecoder", m: int) -> int:
-    """Parts per token of the fused MLP tail at block width ``m``, 0 when the three-launch form
-    runs (wider blocks, fp16 scales, shapes the fused kernels do not take, BONSAI_FUSED_MLP=0)."""
-    if m > 2 or os.environ.get("BONSAI_FUSED_MLP", "1") == "0":
-        return 0
+def fused_plan(model: "BonsaiDecoder", m: int) -> Optional[FusedPlan]:
+    """How a step of width ``m`` runs its layers: with the residual add + RMSNorm + quantisation
+    and the SiLU * up + quantisation folded into the projections (seven launches a layer instead of
+    ten; blocks of one or two tokens), or -- ``None`` -- with the separate producers (wider blocks,
+    shapes the fused kernels do not take, BONSAI_FUSED_STEP=0)."""
+    if m > ops.FUSED_MAX_TOKENS or os.environ.get("BONSAI_FUSED_STEP", "1") == "0":
+        return None
     lw = model.layers[0]
-    if lw.w_gu.bits != lw.w_down.bits or lw.w_gu.weight_scale.dtype != torch.bfloat16:
-        return 0
-    lib = ops.t2_lib() if lw.w_gu.bits == 2 else ops.q1_lib()
-    fn = lib.t2g128_silu_pair_parts if lw.w_gu.bits == 2 else lib.q1g128_silu_pair_parts
-    parts = fn(m, lw.w_gu.out_features, lw.w_gu.in_features)
-    return parts if 0 < parts <= 1024 else 0
+    packed = (lw.wqkv, lw.wo, lw.w_gu, lw.w_down)
+    if len({p.bits for p in packed}) != 1 or any(p.weight_scale.dtype != torch.bfloat16 for p in packed):
+        return None
+    bits = lw.wo.bits
+    plan = FusedPlan(
+        o=ops.fused_parts(ops.EPI_ADD_SUMSQ, m, lw.wo.out_features, lw.wo.in_features, bits=bits),
+        gu=ops.fused_parts(ops.EPI_SILU_PAIR, m, lw.w_gu.out_features, lw.w_gu.in_features, bits=bits),
+        down=ops.fused_parts(ops.EPI_ADD_SUMSQ, m, lw.w_down.out_features, lw.w_down.in_features, bits=bits))
+    if min(plan.o, plan.gu, plan.down) < 1 or max(plan.o, plan.down) > 256 or plan.gu > 1024:
+        return None
+    return plan
+
+
+def _fused(w: PackedLinear, m: int, stream: ctypes.c_void_p, *, act, act_aux, act_kind: int, out,
+           epi: int, act_parts: int = 0, norm_w=None, eps: float = 0.0, residual=None, out_aux=None) -> None:
+    d = ops.FusedGemvDesc(act=act.data_ptr(), act_aux=act_aux.data_ptr(),
+                          norm_weight=norm_w.data_ptr() if norm_w is not None else None,
+                          B=w.weight.data_ptr(), ws=w.weight_scale.data_ptr(), out=out.data_ptr(),
+                          residual=residual.data_ptr() if residual is not None else None,
+                          out_aux=out_aux.data_ptr() if out_aux is not None else None, s_out=None,
+                          eps=eps, M=m, N=w.out_features, K=w.in_features, act_kind=act_kind,
+                          act_parts=act_parts, epi_kind=epi, out_kind=ops.OUT_BF16)
+    fn = ops.t2_lib().t2g128_gemv_fused if w.bits == 2 else ops.q1_lib().q1g128_gemv_fused
+    rc = fn(ctypes.byref(d), stream)
+    if rc != 0:
+        raise RuntimeError(f"{'t2g128' if w.bits == 2 else 'q1g128'}_gemv_fused failed with status {rc} "
+                           f"(act {act_kind}, epilogue {epi}, M={m}, N={w.out_features}, K={w.in_features})")
 
 
 def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tensor, sigma: int,
@@ -505,10 +520,37 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
         if rc != 0:
             raise RuntimeError(f"{what} failed with status {rc}")
 
-    tail_parts = mlp_tail_parts(model, M)
+    plan = fused_plan(model, M)
     h_cur, h_nxt = ws.h[0][:M], ws.h[1][:M]
     torch.index_select(model.embed, 0, io.tokens, out=h_cur)
     for i, lw in enumerate(model.layers):
+        if plan is not None:
+            # seven launches: the element-wise producers ride in the projections on either side;
+            # h_cur already holds the residual stream including the previous layer's MLP
+            if i == 0:
+                check(actq.bonsai_rmsnorm_quant_int8(_vp(h_cur), _vp(lw.input_layernorm), eps,
+                                                     _vp(ws.a_q), _vp(ws.a_s), M, dim, stream),
+                      "bonsai_rmsnorm_quant_int8")
+                _gemv(ws.a_q, ws.a_s, lw.wqkv, ws.xqkv, M, stream)
+            else:
+                _fused(lw.wqkv, M, stream, act=h_cur, act_aux=ws.sumsq, act_kind=ops.ACT_BF16_NORM,
+                       act_parts=plan.down, norm_w=lw.input_layernorm, eps=eps, out=ws.xqkv,
+                       epi=ops.EPI_PLAIN)
+            decode_ops.qk_norm_rope_kv_write(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
+                                             io.positions, ws.q[:M], kv[0, i], kv[1, i],
+                                             args.n_heads, args.n_kv_heads, sigma)
+            decode_ops.decode_attention(ws.q[:M], kv[0, i], kv[1, i], io.meta, ws.attn_scratch, sigma,
+                                        out_q=ws.o_q[:M], out_s=ws.o_s[:M])
+            _fused(lw.wo, M, stream, act=ws.o_q, act_aux=ws.o_s, act_kind=ops.ACT_INT8, out=h_nxt,
+                   epi=ops.EPI_ADD_SUMSQ, residual=h_cur, out_aux=ws.sumsq)
+            h_cur, h_nxt = h_nxt, h_cur
+            _fused(lw.w_gu, M, stream, act=h_cur, act_aux=ws.sumsq, act_kind=ops.ACT_BF16_NORM,
+                   act_parts=plan.o, norm_w=lw.post_attention_layernorm, eps=eps, out=ws.inner,
+                   epi=ops.EPI_SILU_PAIR, out_aux=ws.inner_amax)
+            _fused(lw.w_down, M, stream, act=ws.inner, act_aux=ws.inner_amax, act_kind=ops.ACT_BF16_AMAX,
+                   act_parts=plan.gu, out=h_nxt, epi=ops.EPI_ADD_SUMSQ, residual=h_cur, out_aux=ws.sumsq)
+            h_cur, h_nxt = h_nxt, h_cur
+            continue
         if i == 0:
             check(actq.bonsai_rmsnorm_quant_int8(_vp(h_cur), _vp(lw.input_layernorm), eps,
                                                  _vp(ws.a_q), _vp(ws.a_s), M, dim, stream),
@@ -531,23 +573,23 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
                                                  _vp(ws.f_q), _vp(ws.f_s), M, dim, stream),
               "bonsai_add_rmsnorm_quant_int8")
         h_cur, h_nxt = h_nxt, h_cur
-        if tail_parts:
-            _mlp_tail_fused(lw, ws, M, tail_parts, stream)
-        else:
-            _gemv(ws.f_q, ws.f_s, lw.w_gu, ws.gu, M, stream)
-            check(actq.bonsai_silu_mul_quant_int8(_vp(ws.gu), _vp(ws.i_q), _vp(ws.i_s), M,
-                                                  args.ffn_dim, stream),
-                  "bonsai_silu_mul_quant_int8")
-            _gemv(ws.i_q, ws.i_s, lw.w_down, ws.ffn_out, M, stream)
+        _gemv(ws.f_q, ws.f_s, lw.w_gu, ws.gu, M, stream)
+        check(actq.bonsai_silu_mul_quant_int8(_vp(ws.gu), _vp(ws.i_q), _vp(ws.i_s), M,
+                                              args.ffn_dim, stream),
+              "bonsai_silu_mul_quant_int8")
+        _gemv(ws.i_q, ws.i_s, lw.w_down, ws.ffn_out, M, stream)
+
+    # the last MLP's result: still to be added (ffn_out + h_cur), or already in the stream (fused layers)
+    last_x = ws.ffn_out[logits_start:] if plan is None else h_cur[logits_start:]
+    last_res = _vp(h_cur[logits_start:]) if plan is None else None
 
     rows = logits_end - logits_start
     if head_mode not in ("native", "fp8", "bf16_raw"):
         raise ValueError(f"unknown head_mode {head_mode!r}")
     if head_mode != "native" or model.head is None:
         # projections of the normalised bf16 rows (reference: model.py:1401-1403)
-        check(actq.bonsai_add_rmsnorm_bf16(_vp(ws.ffn_out[logits_start:]), _vp(h_cur[logits_start:]),
-                                           _vp(model.norm), eps, _vp(ws.h_last), _vp(ws.l_n),
-                                           rows, dim, stream),
+        check(actq.bonsai_add_rmsnorm_bf16(_vp(last_x), last_res, _vp(model.norm), eps, _vp(ws.h_last),
+                                           _vp(ws.l_n), rows, dim, stream),
               "bonsai_add_rmsnorm_bf16")
         if head_mode == "fp8":
             if model.head_fp8 is None:
@@ -563,11 +605,15 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
             logits = ws.logits_view(rows, w.shape[0])
             decode_ops.bf16_linear(ws.l_n[:rows], w, logits)
     else:
-        check(actq.bonsai_add_rmsnorm_quant_int8(_vp(ws.ffn_out[logits_start:]),
-                                                 _vp(h_cur[logits_start:]), _vp(model.norm), eps,
-                                                 _vp(ws.h_last), _vp(ws.l_q), _vp(ws.l_s), rows,
-                                                 dim, stream),
-              "bonsai_add_rmsnorm_quant_int8")
+        if plan is None:
+            check(actq.bonsai_add_rmsnorm_quant_int8(_vp(last_x), last_res, _vp(model.norm), eps,
+                                                     _vp(ws.h_last), _vp(ws.l_q), _vp(ws.l_s), rows,
+                                                     dim, stream),
+                  "bonsai_add_rmsnorm_quant_int8")
+        else:
+            check(actq.bonsai_rmsnorm_quant_int8(_vp(last_x), _vp(model.norm), eps, _vp(ws.l_q),
+                                                 _vp(ws.l_s), rows, dim, stream),
+                  "bonsai_rmsnorm_quant_int8")
         logits = ws.logits_view(rows, model.head_rows)
         _gemv(ws.l_q, ws.l_s, model.head, logits, rows, stream)
     # (the attention scratch is free again by now and far larger than the chain needs)

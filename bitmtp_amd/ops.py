@@ -35,11 +35,18 @@ _GEMV_EX_ARGTYPES = [
     ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
     ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
 ]
-# (A, B, inner, s, ws, M, N2, K, amax, stream) and
-# (inner, B, out, ws, M, N, K, amax, parts, s_out, out_kind, stream)
-_SILU_PAIR_ARGTYPES = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p] * 2
-_BF16_ACT_ARGTYPES = ([ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 +
-                      [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p])
+ACT_INT8, ACT_BF16_AMAX, ACT_BF16_NORM = 0, 1, 2
+EPI_PLAIN, EPI_SILU_PAIR, EPI_ADD_SUMSQ = 0, 1, 2
+
+
+class FusedGemvDesc(ctypes.Structure):
+    """``bonsai_fused_gemv`` of include/bonsai_gemv.h."""
+    _fields_ = [("act", ctypes.c_void_p), ("act_aux", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p),
+                ("B", ctypes.c_void_p), ("ws", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("residual", ctypes.c_void_p), ("out_aux", ctypes.c_void_p), ("s_out", ctypes.c_void_p),
+                ("eps", ctypes.c_float), ("M", ctypes.c_int32), ("N", ctypes.c_int32), ("K", ctypes.c_int32),
+                ("act_kind", ctypes.c_int32), ("act_parts", ctypes.c_int32), ("epi_kind", ctypes.c_int32),
+                ("out_kind", ctypes.c_int32)]
 
 
 class GemvDesc(ctypes.Structure):
@@ -100,12 +107,10 @@ def load_t2_kernel() -> None:
     lib.t2g128_last_kernel.restype = ctypes.c_char_p
     lib.t2g128_launch_count.argtypes = []
     lib.t2g128_launch_count.restype = ctypes.c_int
-    lib.t2g128_silu_pair_parts.argtypes = [ctypes.c_int] * 3
-    lib.t2g128_silu_pair_parts.restype = ctypes.c_int
-    lib.t2g128_gemv_silu_pair.argtypes = _SILU_PAIR_ARGTYPES
-    lib.t2g128_gemv_silu_pair.restype = ctypes.c_int
-    lib.t2g128_gemv_bf16_act.argtypes = _BF16_ACT_ARGTYPES
-    lib.t2g128_gemv_bf16_act.restype = ctypes.c_int
+    lib.t2g128_fused_parts.argtypes = [ctypes.c_int] * 4
+    lib.t2g128_fused_parts.restype = ctypes.c_int
+    lib.t2g128_gemv_fused.argtypes = [ctypes.POINTER(FusedGemvDesc), ctypes.c_void_p]
+    lib.t2g128_gemv_fused.restype = ctypes.c_int
     _t2_lib = lib
 
 
@@ -138,12 +143,10 @@ def load_q1_kernel() -> None:
     lib.q1g128_last_kernel.restype = ctypes.c_char_p
     lib.q1g128_launch_count.argtypes = []
     lib.q1g128_launch_count.restype = ctypes.c_int
-    lib.q1g128_silu_pair_parts.argtypes = [ctypes.c_int] * 3
-    lib.q1g128_silu_pair_parts.restype = ctypes.c_int
-    lib.q1g128_gemv_silu_pair.argtypes = _SILU_PAIR_ARGTYPES
-    lib.q1g128_gemv_silu_pair.restype = ctypes.c_int
-    lib.q1g128_gemv_bf16_act.argtypes = _BF16_ACT_ARGTYPES
-    lib.q1g128_gemv_bf16_act.restype = ctypes.c_int
+    lib.q1g128_fused_parts.argtypes = [ctypes.c_int] * 4
+    lib.q1g128_fused_parts.restype = ctypes.c_int
+    lib.q1g128_gemv_fused.argtypes = [ctypes.POINTER(FusedGemvDesc), ctypes.c_void_p]
+    lib.q1g128_gemv_fused.restype = ctypes.c_int
     _q1_lib = lib
 
 
@@ -402,98 +405,120 @@ def packed_gemv_ex(a_int8: torch.Tensor, b_packed: torch.Tensor, s: Optional[tor
     return out
 
 
-FUSED_MLP_MAX_TOKENS = 2
+FUSED_MAX_TOKENS = 2
 
 
-def silu_pair_parts(m: int, n2: int, k: int, *, bits: int) -> int:
-    """Maxima per token that :func:`packed_gemv_silu_pair` writes for this shape (the number
-    of workgroups of its launch); 0 when the shape is not taken."""
-    fn = t2_lib().t2g128_silu_pair_parts if bits == 2 else q1_lib().q1g128_silu_pair_parts
-    parts = fn(m, n2, k)
+def fused_parts(epi: int, m: int, n: int, k: int, *, bits: int) -> int:
+    """Parts per token that a fused launch with epilogue ``epi`` writes for this shape (the
+    number of workgroups of that launch); 0 when the shape is not taken."""
+    fn = t2_lib().t2g128_fused_parts if bits == 2 else q1_lib().q1g128_fused_parts
+    parts = fn(epi, m, n, k)
     if parts < -1:
-        raise RuntimeError(f"silu_pair_parts: native set-up failed with status {-parts}")
+        raise RuntimeError(f"fused_parts: native set-up failed with status {-parts}")
     return max(parts, 0)
 
 
-def packed_gemv_silu_pair(a_int8: torch.Tensor, b_gate_up: torch.Tensor, s: torch.Tensor,
-                          ws: torch.Tensor, *, bits: int, inner: Optional[torch.Tensor] = None,
-                          amax: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, int]:
-    """The merged gate|up projection (rows ``[gate; up]``) of one or two quantised tokens with
-    ``inner = bf16(bf16(silu(gate)) * up)`` computed in its epilogue: returns ``(inner bf16
-    [M, F], amax bf16 [M, ld], parts)`` where ``amax[m, :parts]`` holds max ``|inner[m]|`` of
-    each workgroup of the launch.  Together with :func:`packed_gemv_bf16_act` it stands for
-    projection, SiLU * up + quantisation (reference: model.py:1059-1061) and projection, with
-    the same bits."""
-    kind = "t2g128" if bits == 2 else "q1"
-    if a_int8.dim() != 2:
-        raise ValueError(f"{kind}: expected rank-2 activation")
-    _validate_packed_inputs(a_int8, b_gate_up, s, ws, kind=kind, bits=bits,
-                            activation_dtype=torch.int8, scale_dtypes=(torch.bfloat16,))
-    m, n2, k = a_int8.shape[0], b_gate_up.shape[0], b_gate_up.shape[1] * (8 // bits)
-    if m > FUSED_MLP_MAX_TOKENS or n2 % 2:
-        raise RuntimeError(f"{kind}: the fused MLP tail takes one or two tokens and an even row count")
-    dev = a_int8.device
-    with torch.cuda.device(dev):
-        parts = silu_pair_parts(m, n2, k, bits=bits)
-        if parts == 0:
-            raise RuntimeError(f"{kind}: shape not taken by the fused MLP tail (M={m}, N={n2}, K={k})")
-        ld = (parts + 7) // 8 * 8
-        if inner is None:
-            inner = torch.empty(m, n2 // 2, dtype=torch.bfloat16, device=dev)
-        if amax is None:
-            amax = torch.empty(m, ld, dtype=torch.bfloat16, device=dev)
-        if (tuple(inner.shape) != (m, n2 // 2) or inner.dtype != torch.bfloat16 or not inner.is_contiguous()
-                or amax.dtype != torch.bfloat16 or amax.numel() < m * ld or not amax.is_contiguous()
-                or inner.device != dev or amax.device != dev):
-            raise RuntimeError(f"{kind}: inner must be bf16 [{m}, {n2 // 2}] and amax bf16 with at least "
-                               f"{m * ld} elements, contiguous, on {dev}")
-        fn = t2_lib().t2g128_gemv_silu_pair if bits == 2 else q1_lib().q1g128_gemv_silu_pair
-        rc = fn(_ptr(a_int8), _ptr(b_gate_up), _ptr(inner), _ptr(s), _ptr(ws), m, n2, k, _ptr(amax),
-                _stream(dev))
-    if rc != 0:
-        raise RuntimeError(f"{kind}: native launch failed with status {rc} (M={m}, N={n2}, K={k})")
-    return inner, amax, parts
+def _amax_ld(parts: int) -> int:
+    return (parts + 7) // 8 * 8
 
 
-def packed_gemv_bf16_act(inner: torch.Tensor, b_packed: torch.Tensor, ws: torch.Tensor,
-                         amax: torch.Tensor, parts: int, *, bits: int, out_kind: int = OUT_BF16,
-                         out: Optional[torch.Tensor] = None,
-                         s_out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Projection of bf16 activations ``inner [M, K]`` (one or two tokens) that are quantised
-    per token while they are staged, with ``s = fl(fl(1 / max(amax, 1e-5)) * 127)`` taken from
-    the ``parts`` maxima per token that :func:`packed_gemv_silu_pair` left in ``amax``; ``s_out``
-    (fp32 [M]) receives the multipliers when given."""
+def packed_gemv_fused(act: torch.Tensor, b_packed: torch.Tensor, ws: torch.Tensor, *, bits: int,
+                      s: Optional[torch.Tensor] = None, amax: Optional[torch.Tensor] = None,
+                      sumsq: Optional[torch.Tensor] = None, parts: int = 0,
+                      norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                      epi: int = EPI_PLAIN, residual: Optional[torch.Tensor] = None,
+                      out: Optional[torch.Tensor] = None, out_aux: Optional[torch.Tensor] = None,
+                      s_out: Optional[torch.Tensor] = None, out_kind: int = OUT_BF16):
+    """One projection of a one- or two-token decode step with the element-wise work of its
+    neighbours folded in (``*_gemv_fused`` of include/bonsai_gemv.h).
+
+    What it reads: ``s`` given -- int8 ``act`` with its multipliers, as :func:`packed_gemv_ex`;
+    ``amax`` given -- bf16 ``act`` quantised on the fly from the ``parts`` maxima per token a
+    SiLU-pair launch left; ``sumsq`` given -- bf16 ``act`` = residual stream, RMS-normalised with
+    ``norm_weight`` / ``eps`` from the ``parts`` sums of squares an add launch left, then quantised.
+    What it stores (``epi``): the plain result; ``EPI_SILU_PAIR`` -- ``bf16(bf16(silu(gate)) *
+    up)`` of merged rows ``[gate; up]`` plus maxima; ``EPI_ADD_SUMSQ`` -- ``bf16(residual +
+    bf16(y))`` plus sums of squares.  Returns ``(out, out_aux, out_parts)``.
+    Reference: the helpers between the projections, model.py:307-336 and :1058-1061."""
     kind = "t2g128" if bits == 2 else "q1"
-    if inner.dim() != 2 or inner.dtype != torch.bfloat16 or not inner.is_contiguous() or not inner.is_cuda:
-        raise RuntimeError(f"{kind}: expected contiguous rank-2 bf16 CUDA activations")
-    m, n, k = inner.shape[0], b_packed.shape[0], b_packed.shape[1] * (8 // bits)
-    if inner.shape[1] != k or m > FUSED_MLP_MAX_TOKENS:
-        raise RuntimeError(f"{kind}: inner must be [M <= {FUSED_MLP_MAX_TOKENS}, {k}]")
+    given = [x is not None for x in (s, amax, sumsq)]
+    if sum(given) != 1:
+        raise ValueError(f"{kind}: exactly one of s, amax, sumsq selects what the launch reads")
+    act_kind = ACT_INT8 if s is not None else (ACT_BF16_AMAX if amax is not None else ACT_BF16_NORM)
+    if epi not in (EPI_PLAIN, EPI_SILU_PAIR, EPI_ADD_SUMSQ):
+        raise ValueError("bad epi")
+    if act.dim() != 2 or b_packed.dim() != 2:
+        raise ValueError(f"{kind}: expected rank-2 activation and rank-2 weight")
+    m, n, k = act.shape[0], b_packed.shape[0], b_packed.shape[1] * (8 // bits)
+    dev = act.device
+    want_act = torch.int8 if act_kind == ACT_INT8 else torch.bfloat16
+    if act.dtype != want_act or act.shape[1] != k or b_packed.dtype != torch.int8:
+        raise RuntimeError(f"{kind}: activations must be {want_act} [M, {k}] and the weights packed int8")
+    if m < 1 or m > FUSED_MAX_TOKENS:
+        raise RuntimeError(f"{kind}: the fused forms take one or two tokens")
     if ws.dtype != torch.bfloat16 or tuple(ws.shape) != (n, k // 128):
         raise RuntimeError(f"{kind}: weight scales must be bf16 [{n}, {k // 128}]")
-    if out_kind not in (OUT_BF16, OUT_F32):
-        raise ValueError("bad out_kind")
-    ld = (parts + 7) // 8 * 8
-    if amax.dtype != torch.bfloat16 or amax.numel() < m * ld or parts < 1 or not amax.is_contiguous():
-        raise RuntimeError(f"{kind}: amax must be contiguous bf16 with at least {m * ld} elements")
-    dev = inner.device
-    dtype = torch.bfloat16 if out_kind == OUT_BF16 else torch.float32
-    if out is None:
-        out = torch.empty(m, n, dtype=dtype, device=dev)
-    elif tuple(out.shape) != (m, n) or out.dtype != dtype or out.device != dev or not out.is_contiguous():
-        raise RuntimeError(f"{kind}: out must be a contiguous {dtype} tensor of shape {(m, n)} on {dev}")
-    if s_out is not None and (s_out.dtype != torch.float32 or s_out.numel() < m or s_out.device != dev):
-        raise RuntimeError(f"{kind}: s_out must be fp32 with at least {m} elements on {dev}")
-    for t in (b_packed, ws, amax):
-        if t.device != dev:
-            raise RuntimeError(f"{kind}: all operands must be on {dev}")
-    fn = t2_lib().t2g128_gemv_bf16_act if bits == 2 else q1_lib().q1g128_gemv_bf16_act
+    aux = s if s is not None else (amax if amax is not None else sumsq)
+    if act_kind == ACT_INT8:
+        if s.dtype != torch.float32 or s.numel() != m:
+            raise RuntimeError(f"{kind}: activation scales must be float32 with one value per row")
+    elif act_kind == ACT_BF16_AMAX:
+        if amax.dtype != torch.bfloat16 or parts < 1 or amax.numel() < m * _amax_ld(parts):
+            raise RuntimeError(f"{kind}: amax must be bf16 with at least {m * _amax_ld(parts)} elements")
+    else:
+        if sumsq.dtype != torch.float64 or parts < 1 or sumsq.numel() < m * parts:
+            raise RuntimeError(f"{kind}: sumsq must be float64 with at least {m * parts} elements")
+        if norm_weight is None or norm_weight.dtype != torch.bfloat16 or norm_weight.numel() != k:
+            raise RuntimeError(f"{kind}: norm_weight must be bf16 [{k}]")
+    out_parts = 0
     with torch.cuda.device(dev):
-        rc = fn(_ptr(inner), _ptr(b_packed), _ptr(out), _ptr(ws), m, n, k, _ptr(amax), parts,
-                _ptr(s_out), out_kind, _stream(dev))
+        if epi != EPI_PLAIN:
+            if out_kind != OUT_BF16:
+                raise ValueError(f"{kind}: this epilogue stores bf16")
+            if epi == EPI_SILU_PAIR and n % 2:
+                raise RuntimeError(f"{kind}: merged gate|up rows must be even in number")
+            out_parts = fused_parts(epi, m, n, k, bits=bits)
+            if out_parts == 0:
+                raise RuntimeError(f"{kind}: shape not taken by the fused forms (M={m}, N={n}, K={k})")
+        n_out = n // 2 if epi == EPI_SILU_PAIR else n
+        dtype = torch.float32 if (epi == EPI_PLAIN and out_kind == OUT_F32) else torch.bfloat16
+        if epi == EPI_PLAIN and out_kind not in (OUT_BF16, OUT_F32):
+            raise ValueError("bad out_kind")
+        if out is None:
+            out = torch.empty(m, n_out, dtype=dtype, device=dev)
+        elif tuple(out.shape) != (m, n_out) or out.dtype != dtype or not out.is_contiguous():
+            raise RuntimeError(f"{kind}: out must be a contiguous {dtype} tensor of shape {(m, n_out)}")
+        if epi == EPI_SILU_PAIR:
+            need, adt = m * _amax_ld(out_parts), torch.bfloat16
+        elif epi == EPI_ADD_SUMSQ:
+            need, adt = m * out_parts, torch.float64
+            if residual is None or residual.dtype != torch.bfloat16 or tuple(residual.shape) != (m, n):
+                raise RuntimeError(f"{kind}: residual must be bf16 [{m}, {n}]")
+        else:
+            need, adt = 0, None
+        if need:
+            if out_aux is None:
+                out_aux = torch.empty(need, dtype=adt, device=dev)
+            elif out_aux.dtype != adt or out_aux.numel() < need or not out_aux.is_contiguous():
+                raise RuntimeError(f"{kind}: out_aux must be contiguous {adt} with at least {need} elements")
+        if s_out is not None and (act_kind == ACT_INT8 or s_out.dtype != torch.float32 or s_out.numel() < m):
+            raise RuntimeError(f"{kind}: s_out is fp32 [M] and only for bf16 activations")
+        tensors = [t for t in (act, b_packed, ws, aux, norm_weight, residual, out, out_aux, s_out) if t is not None]
+        if not all(t.is_cuda and t.is_contiguous() and t.device == dev for t in tensors):
+            raise RuntimeError(f"{kind}: operands must be contiguous tensors on {dev}")
+        d = FusedGemvDesc(act=act.data_ptr(), act_aux=aux.data_ptr(),
+                          norm_weight=norm_weight.data_ptr() if norm_weight is not None else None,
+                          B=b_packed.data_ptr(), ws=ws.data_ptr(), out=out.data_ptr(),
+                          residual=residual.data_ptr() if residual is not None else None,
+                          out_aux=out_aux.data_ptr() if out_aux is not None else None,
+                          s_out=s_out.data_ptr() if s_out is not None else None,
+                          eps=float(eps), M=m, N=n, K=k, act_kind=act_kind, act_parts=int(parts),
+                          epi_kind=epi, out_kind=out_kind)
+        fn = t2_lib().t2g128_gemv_fused if bits == 2 else q1_lib().q1g128_gemv_fused
+        rc = fn(ctypes.byref(d), _stream(dev))
     if rc != 0:
         raise RuntimeError(f"{kind}: native launch failed with status {rc} (M={m}, N={n}, K={k})")
-    return out
+    return out, out_aux, out_parts
 
 
 def packed_gemv_grouped(problems: Sequence[Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor],

@@ -115,41 +115,66 @@ int t2g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, 
 int q1g128_gemv_grouped(const bonsai_gemv_desc *descs, int count, int out_kind, int scale_kind,
                         void *stream);
 
-/* ---- the MLP tail as two launches (blocks of one or two tokens) ---------------------- */
-/* No counterpart in the reference, which runs gate|up projection, a torch.compile'd helper
- * (inner = silu(gate) * up, then `quant_input`; src/bonsai_sft/gpu/model.py:1058-1061) and
- * the down projection as three launches.  For one or two tokens every launch of a decode step
- * costs about as much as the projection itself, so the middle one is folded into its
- * neighbours; the operations and their rounding points are those of the three-launch form
- * (bonsai_silu_mul_quant_int8 between two *_gemv_ex calls with BONSAI_SCALE_BF16 on the dot4
- * kernels) and the results are the same bits.
+/* ---- decode steps of one or two tokens without their element-wise launches ------------ */
+/* No counterpart in the reference, which runs a torch.compile'd helper between two projections:
+ * residual add + RMSNorm + `quant_input` (src/bonsai_sft/gpu/model.py:307-336, called at
+ * :977,1006,1058) or silu(gate) * up + `quant_input` (model.py:1058-1061).  For one or two tokens
+ * every launch of a decode step costs about as much as a projection, so these helpers are folded
+ * into the projections on either side.  A row-wide value the helper needs (max |x| for the
+ * quantisation, sum x^2 for the norm) is left by the projection that produces the row as one
+ * PART per workgroup and token, and added up by every wave of the projection that consumes it.
  *
- * *_gemv_silu_pair: B holds the merged rows [gate (F rows); up (F rows)], N2 = 2 F.  Computes
- *   both projections of A (int8 [M, K], multipliers s) and writes
- *   inner = bf16(bf16(silu(gate)) * up) as bf16 [M, F]; the bf16 rounded projections themselves
- *   are not stored.  amax (bf16, 16-byte aligned, [M, ld] with ld = parts rounded up to a
- *   multiple of 8) receives max |inner[m]| over the columns of each of the launch's `parts`
- *   workgroups; every element of [M, ld] is written.  parts = *_silu_pair_parts(M, N2, K)
- *   depends on the shape only (at most 1024).
- * *_gemv_bf16_act: projects inner (bf16 [M, K]) after quantising it per token while staging:
- *   s[m] = fl(fl(1 / max(max_p amax[m][p], 1e-5)) * 127), q = clamp(rne(fl(inner * s)), -128, 127),
- *   as bonsai_act_quant_int8 would; out is bf16 or fp32 [M, N] (BONSAI_OUT_BF16 / _F32);
- *   s_out (fp32 [M], may be NULL) receives the multipliers.
- * M <= 2; bf16 weight scales; other operands as for *_gemv_ex.  *_silu_pair_parts returns -1
- * for a shape these kernels do not take (the caller then uses the three-launch form), -2 / -3
- * for the set-up failures BONSAI_ERR_LAUNCH / BONSAI_ERR_NOT_INIT. */
-int t2g128_silu_pair_parts(int M, int N2, int K);
-int q1g128_silu_pair_parts(int M, int N2, int K);
-int t2g128_gemv_silu_pair(const int8_t *A, const uint8_t *B, void *inner, const float *s,
-                          const void *ws, int M, int N2, int K, void *amax, void *stream);
-int q1g128_gemv_silu_pair(const int8_t *A, const uint8_t *B, void *inner, const float *s,
-                          const void *ws, int M, int N2, int K, void *amax, void *stream);
-int t2g128_gemv_bf16_act(const void *inner, const uint8_t *B, void *out, const void *ws, int M,
-                         int N, int K, const void *amax, int parts, float *s_out, int out_kind,
-                         void *stream);
-int q1g128_gemv_bf16_act(const void *inner, const uint8_t *B, void *out, const void *ws, int M,
-                         int N, int K, const void *amax, int parts, float *s_out, int out_kind,
-                         void *stream);
+ * epi_kind (what the launch stores):
+ *   BONSAI_EPI_PLAIN      out = bf16 / fp32 [M, N] as *_gemv_ex (out_kind BONSAI_OUT_BF16 / _F32)
+ *   BONSAI_EPI_SILU_PAIR  B holds the merged rows [gate (N/2 rows); up (N/2 rows)]:
+ *                         out = bf16(bf16(silu(gate)) * up) as bf16 [M, N/2]; out_aux = bf16
+ *                         [M, ld], ld = parts rounded up to a multiple of 8, 16-byte aligned:
+ *                         max |out[m]| over the columns of each workgroup; all of [M, ld] is written
+ *   BONSAI_EPI_ADD_SUMSQ  out = bf16(residual + bf16(y)) as bf16 [M, N] (residual bf16 [M, N], may
+ *                         be the buffer a later launch overwrites but not `out`); out_aux = fp64
+ *                         [M, parts]: sum of out[m]^2 over the columns of each workgroup
+ *   parts = *_fused_parts(epi_kind, M, N, K): the workgroups of that launch; depends on the shape only.
+ * act_kind (what the launch reads):
+ *   BONSAI_ACT_INT8       act int8 [M, K], act_aux = fp32 s[M], as *_gemv_ex
+ *   BONSAI_ACT_BF16_AMAX  act bf16 [M, K], act_aux = the bf16 maxima an EPI_SILU_PAIR launch left
+ *                         (act_parts of them per token): s[m] = fl(fl(1 / max(amax, 1e-5)) * 127),
+ *                         q = clamp(rne(fl(act * s)), -128, 127), as bonsai_act_quant_int8
+ *   BONSAI_ACT_BF16_NORM  act = h bf16 [M, K], act_aux = the fp64 sums an EPI_ADD_SUMSQ launch left
+ *                         (act_parts per token), norm_weight bf16 [K], eps:
+ *                         var = fp32(sum) / K, x = bf16(w * bf16(h * rsqrt(var + eps))), then as
+ *                         BONSAI_ACT_BF16_AMAX on max |x|: bonsai_rmsnorm_quant_int8 without its launch
+ *   s_out (fp32 [M], may be NULL; BF16 kinds only) receives the multipliers.
+ * The operations and rounding points are those of the stand-alone producers between *_gemv_ex
+ * calls on the dot4 kernels, so the results are the same bits; the fp64 sum of squares alone is
+ * added up in another order (per workgroup, then over the parts), which can show only where two
+ * fp64 roundings differ AND the fp32 conversion of the sum straddles a rounding boundary.
+ * M <= 2, bf16 weight scales, operands aligned as for *_gemv_ex (act_aux / out_aux: 16 bytes for
+ * maxima, 8 for sums).  *_fused_parts returns -1 for a shape these kernels do not take (use the
+ * separate launches), -2 / -3 for the set-up failures BONSAI_ERR_LAUNCH / BONSAI_ERR_NOT_INIT. */
+#define BONSAI_ACT_INT8 0
+#define BONSAI_ACT_BF16_AMAX 1
+#define BONSAI_ACT_BF16_NORM 2
+#define BONSAI_EPI_PLAIN 0
+#define BONSAI_EPI_SILU_PAIR 1
+#define BONSAI_EPI_ADD_SUMSQ 2
+typedef struct bonsai_fused_gemv {
+    const void *act;
+    const void *act_aux;
+    const void *norm_weight; /* BONSAI_ACT_BF16_NORM only */
+    const uint8_t *B;        /* packed weights [N, K/4] (T2) or [N, K/8] (Q1) */
+    const void *ws;          /* bf16 [N, K/128] */
+    void *out;
+    const void *residual;    /* BONSAI_EPI_ADD_SUMSQ only */
+    void *out_aux;           /* BONSAI_EPI_SILU_PAIR / _ADD_SUMSQ */
+    float *s_out;
+    float eps;
+    int32_t M, N, K;
+    int32_t act_kind, act_parts, epi_kind, out_kind;
+} bonsai_fused_gemv;
+int t2g128_fused_parts(int epi_kind, int M, int N, int K);
+int q1g128_fused_parts(int epi_kind, int M, int N, int K);
+int t2g128_gemv_fused(const bonsai_fused_gemv *d, void *stream);
+int q1g128_gemv_fused(const bonsai_fused_gemv *d, void *stream);
 
 /* One-time set-up for the current device (raises the kernels' dynamic-LDS
  * limit).  Called implicitly by the first launch; call it explicitly before
