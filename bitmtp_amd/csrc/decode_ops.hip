@@ -76,6 +76,30 @@ struct RopeArgs {
     int M, n_heads, n_kv, slots, write_slot, max_pos;
 };
 
+// RMSNorm + RoPE of one 128-wide head row by one wave: lane i holds the pair (i, i + 64) in
+// (r0, r1) and receives the finished pair in (o0b, o1b) as bf16 bits.
+__device__ __forceinline__ void qk_norm_rope_row(uint32_t r0, uint32_t r1, const uint16_t *w,
+                                                 const uint16_t *cos_t, const uint16_t *sin_t, int pos,
+                                                 int max_pos, float eps, int lane, uint32_t &o0b,
+                                                 uint32_t &o1b) {
+    const float f0 = bf16_bits_to_f32(r0), f1 = bf16_bits_to_f32(r1);
+    const double ss = bonsai_wave::sum64((double)(f0 * f0) + (double)(f1 * f1));
+    const float var = (float)ss / (float)kHd;
+    const float rs = 1.0f / sqrtf(var + eps);
+    const float n0 = bf16_round(bf16_bits_to_f32(w[lane]) * bf16_round(f0 * rs));
+    const float n1 = bf16_round(bf16_bits_to_f32(w[lane + 64]) * bf16_round(f1 * rs));
+    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+    const uint16_t *cr = cos_t + (size_t)pos * kHd;
+    const uint16_t *sr = sin_t + (size_t)pos * kHd;
+    const float c0 = bf16_bits_to_f32(cr[lane]), c1 = bf16_bits_to_f32(cr[lane + 64]);
+    const float s0 = bf16_bits_to_f32(sr[lane]), s1 = bf16_bits_to_f32(sr[lane + 64]);
+    // rotate_half(n) = [-n_hi, n_lo]
+    const float o0 = bf16_round(bf16_round(n0 * c0) + bf16_round(-n1 * s0));
+    const float o1 = bf16_round(bf16_round(n1 * c1) + bf16_round(n0 * s1));
+    o0b = f32_to_bf16_bits(o0);
+    o1b = f32_to_bf16_bits(o1);
+}
+
 __global__ void __launch_bounds__(256)
 qk_norm_rope_kernel(const uint16_t *pxqkv, const uint16_t *pqw, const uint16_t *pkw,
                     const uint16_t *pcos, const uint16_t *psin, const int32_t *ppos,
@@ -100,28 +124,13 @@ qk_norm_rope_kernel(const uint16_t *pxqkv, const uint16_t *pqw, const uint16_t *
         return;
     }
     const bool is_q = head < a.n_heads;
-    const uint16_t *w = is_q ? a.qw : a.kw;
-    const float f0 = bf16_bits_to_f32(r0), f1 = bf16_bits_to_f32(r1);
-    const double ss = bonsai_wave::sum64((double)(f0 * f0) + (double)(f1 * f1));
-    const float var = (float)ss / (float)kHd;
-    const float rs = 1.0f / sqrtf(var + a.eps);
-    const float n0 = bf16_round(bf16_bits_to_f32(w[lane]) * bf16_round(f0 * rs));
-    const float n1 = bf16_round(bf16_bits_to_f32(w[lane + 64]) * bf16_round(f1 * rs));
-
-    int pos = a.positions[m];
-    pos = pos < 0 ? 0 : (pos >= a.max_pos ? a.max_pos - 1 : pos);
-    const uint16_t *cr = a.cos_t + (size_t)pos * kHd;
-    const uint16_t *sr = a.sin_t + (size_t)pos * kHd;
-    const float c0 = bf16_bits_to_f32(cr[lane]), c1 = bf16_bits_to_f32(cr[lane + 64]);
-    const float s0 = bf16_bits_to_f32(sr[lane]), s1 = bf16_bits_to_f32(sr[lane + 64]);
-    // rotate_half(n) = [-n_hi, n_lo]
-    const float o0 = bf16_round(bf16_round(n0 * c0) + bf16_round(-n1 * s0));
-    const float o1 = bf16_round(bf16_round(n1 * c1) + bf16_round(n0 * s1));
-
+    uint32_t o0, o1;
+    qk_norm_rope_row(r0, r1, is_q ? a.qw : a.kw, a.cos_t, a.sin_t, a.positions[m], a.max_pos, a.eps,
+                     lane, o0, o1);
     uint16_t *dst = is_q ? a.q_out + ((size_t)m * a.n_heads + head) * kHd
                          : a.k_layer + ((size_t)(head - a.n_heads) * a.slots + a.write_slot + m) * kHd;
-    dst[lane] = (uint16_t)f32_to_bf16_bits(o0);
-    dst[lane + 64] = (uint16_t)f32_to_bf16_bits(o1);
+    dst[lane] = (uint16_t)o0;
+    dst[lane + 64] = (uint16_t)o1;
 }
 
 // ---------------------------------------------------------------------------
@@ -303,11 +312,32 @@ __host__ __device__ inline int attn_chunks_per_part(int live_chunks, int parts) 
     return (live_chunks + parts - 1) / parts;
 }
 
+// ROPE: the launch takes the merged q|k|v projection instead of finished q rows and does the work
+// of qk_norm_rope_kernel itself, for blocks of at most kRopeFusedMaxWidth tokens (a decode step
+// of one token spends as long on that launch as on this one).  Every workgroup derives the q rows
+// of its pair tile -- one wave per (token, head) row, the very arithmetic of qk_norm_rope_kernel --
+// and hands them to its waves through LDS; a workgroup whose chunks reach the block's own rows
+// (logical index >= cache_len) derives those K rows the same way and takes the V rows from the
+// projection, never from the cache, so no workgroup uses what another one writes; the workgroup
+// of pair tile 0 that owns a row's chunk also writes it to the cache for the steps to come.
+constexpr int kRopeFusedMaxWidth = 2;
+
+struct RopeIn {
+    const uint16_t *qw, *kw, *cos_t, *sin_t;
+    const int32_t *positions;
+    float eps;
+    int max_pos;
+};
+
+template <bool ROPE>
 __global__ void __launch_bounds__(kAttnWaves * 64)
-attn_mfma_kernel(const uint16_t *q, const uint16_t *k_layer, const uint16_t *v_layer,
+attn_mfma_kernel(const uint16_t *q, uint16_t *k_layer, uint16_t *v_layer,
                  const int32_t *meta, float *part_out, float scale_log2e, int M, int n_heads,
-                 int n_kv, int G, int slots, int sigma, int parts) {
+                 int n_kv, int G, int slots, int sigma, int parts, const RopeIn rope) {
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kChunk * kVPitch];
+    __shared__ __attribute__((aligned(16))) uint16_t q_new[ROPE ? kPairTile : 1][kHd];
+    __shared__ __attribute__((aligned(16))) uint16_t k_new[ROPE ? kRopeFusedMaxWidth : 1][kHd];
+    __shared__ __attribute__((aligned(16))) uint16_t v_new[ROPE ? kRopeFusedMaxWidth : 1][kHd];
     __shared__ __attribute__((aligned(16))) unsigned char p_lds[kPairTile * kPPitch];
     __shared__ __attribute__((aligned(16))) float st_max[kAttnWaves][kPairTile];
     __shared__ __attribute__((aligned(16))) float st_sum[kAttnWaves][kPairTile];
@@ -330,16 +360,6 @@ attn_mfma_kernel(const uint16_t *q, const uint16_t *k_layer, const uint16_t *v_l
     const int c_end = min(c_begin + cpw, live_chunks);
     const int pairs_total = M * G;
 
-    // A operand of S: this lane's pair (tile row `col`), dims 32 j + 8 kb .. + 8
-    uint4 qreg[4];
-    {
-        const int qp = min(pt * kPairTile + col, pairs_total - 1);
-        const int qm = qp / G, qg = qp - qm * G;
-        const uint4 *qrow =
-            reinterpret_cast<const uint4 *>(q + ((size_t)qm * n_heads + kvh * G + qg) * kHd);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) qreg[j] = qrow[4 * j + kb];
-    }
     // the four pairs whose results this lane holds (D layout: tile rows 4 kb + r)
     bool valid[4];
     int row_of[4], head_of[4];
@@ -395,13 +415,102 @@ attn_mfma_kernel(const uint16_t *q, const uint16_t *k_layer, const uint16_t *v_l
         cr.v3 = v_row(3);
         return cr;
     };
+    // ROPE: the block's own rows come from LDS (uniform branch), whatever the cache slot held
+    auto own_chunk_rows = [&](ChunkRegs &cr, int c) {
+        const int t0 = c * kChunk + 16 * w;
+        if (ROPE && (c + 1) * kChunk > cache_len) {
+            {
+                const int t = min(t0 + col, total - 1);
+                const uint4 *kn = reinterpret_cast<const uint4 *>(k_new[min(max(t - cache_len, 0), M - 1)]);
+                const uint4 n0 = kn[kb], n1 = kn[4 + kb], n2 = kn[8 + kb], n3 = kn[12 + kb];
+                if (t >= cache_len) {
+                    cr.k0 = n0;
+                    cr.k1 = n1;
+                    cr.k2 = n2;
+                    cr.k3 = n3;
+                }
+            }
+            auto v_own = [&](int i, uint4 &dst) {
+                const int t = min(t0 + 4 * i + kb, total - 1);
+                const uint4 n = reinterpret_cast<const uint4 *>(v_new[min(max(t - cache_len, 0), M - 1)])[col];
+                if (t >= cache_len) dst = n;
+            };
+            v_own(0, cr.v0);
+            v_own(1, cr.v1);
+            v_own(2, cr.v2);
+            v_own(3, cr.v3);
+        }
+    };
 
+    // the first chunk's loads travel while the q rows are fetched or derived
     ChunkRegs cur = load_chunk(c_begin);
+    // ROPE: `q` is the merged projection [M][n_heads + 2 n_kv][128]
+    if constexpr (ROPE) {
+        const bool own_rows = c_end * kChunk > cache_len;  // this workgroup reaches the block's rows
+        const int total_heads = n_heads + 2 * n_kv;
+        const int n_q = min(kPairTile, pairs_total - pt * kPairTile);
+        const int n_jobs = n_q + (own_rows ? M : 0);
+        for (int job = w; job < n_jobs; job += kAttnWaves) {
+            const bool is_q = job < n_q;
+            int m, src_head;
+            if (is_q) {
+                const int qp = pt * kPairTile + job;
+                m = qp / G;
+                src_head = kvh * G + (qp - m * G);
+            } else {
+                m = job - n_q;
+                src_head = n_heads + kvh;
+            }
+            const uint16_t *x = q + ((size_t)m * total_heads + src_head) * kHd;
+            uint32_t o0, o1;
+            qk_norm_rope_row(x[lane], x[lane + 64], is_q ? rope.qw : rope.kw, rope.cos_t, rope.sin_t,
+                             rope.positions[m], rope.max_pos, rope.eps, lane, o0, o1);
+            uint16_t *dst = is_q ? q_new[job] : k_new[m];
+            dst[lane] = (uint16_t)o0;
+            dst[lane + 64] = (uint16_t)o1;
+            if (!is_q) {
+                const uint16_t *xv = q + ((size_t)m * total_heads + n_heads + n_kv + kvh) * kHd;
+                const uint16_t v0 = xv[lane], v1 = xv[lane + 64];
+                v_new[m][lane] = v0;
+                v_new[m][lane + 64] = v1;
+                // the cache row, once: by the workgroup of pair tile 0 that owns the row's chunk
+                const int c_row = (cache_len + m) / kChunk;
+                if (pt == 0 && c_row >= c_begin && c_row < c_end) {
+                    uint16_t *kd = k_layer + ((size_t)kvh * slots + sigma + m) * kHd;
+                    uint16_t *vd = v_layer + ((size_t)kvh * slots + sigma + m) * kHd;
+                    kd[lane] = (uint16_t)o0;
+                    kd[lane + 64] = (uint16_t)o1;
+                    vd[lane] = v0;
+                    vd[lane + 64] = v1;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // A operand of S: this lane's pair (tile row `col`), dims 32 j + 8 kb .. + 8
+    uint4 qreg[4];
+    if constexpr (ROPE) {
+        const int n_q = min(kPairTile, pairs_total - pt * kPairTile);
+        const uint4 *qrow = reinterpret_cast<const uint4 *>(q_new[min(col, n_q - 1)]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qreg[j] = qrow[4 * j + kb];
+    } else {
+        const int qp = min(pt * kPairTile + col, pairs_total - 1);
+        const int qm = qp / G, qg = qp - qm * G;
+        const uint4 *qrow =
+            reinterpret_cast<const uint4 *>(q + ((size_t)qm * n_heads + kvh * G + qg) * kHd);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qreg[j] = qrow[4 * j + kb];
+    }
+    own_chunk_rows(cur, c_begin);
     for (int c = c_begin; c < c_end; ++c) {
         const int t0 = c * kChunk + 16 * w;  // this wave's 16 slots
         // the next chunk's loads go out before this one is worked on (uniform branch)
         ChunkRegs nxt = cur;
-        if (c + 1 < c_end) nxt = load_chunk(c + 1);
+        if (c + 1 < c_end) {
+            nxt = load_chunk(c + 1);
+            own_chunk_rows(nxt, c + 1);
+        }
         const uint4 kreg[4] = {cur.k0, cur.k1, cur.k2, cur.k3};
         const uint4 vreg0 = cur.v0, vreg1 = cur.v1, vreg2 = cur.v2, vreg3 = cur.v3;
 
@@ -1316,10 +1425,12 @@ extern "C" int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int
     return (int64_t)M * n_heads * n_chunks * kPartStride * (int64_t)sizeof(float);
 }
 
-extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const void *v_layer,
-                                       const int32_t *meta, void *scratch, void *out_bf16,
-                                       int8_t *out_q, float *out_s, float scale, int M, int n_heads,
-                                       int n_kv, int slots, int sigma, void *stream) {
+// Shared body of the two attention entry points.  `rope` non-null: `q` is the merged q|k|v
+// projection and the chunk pass does the work of bonsai_qk_norm_rope_kv_write as well.
+static int launch_attention(const void *q, void *k_layer, void *v_layer, const int32_t *meta,
+                            void *scratch, void *out_bf16, int8_t *out_q, float *out_s, float scale,
+                            int M, int n_heads, int n_kv, int slots, int sigma, const RopeIn *rope,
+                            hipStream_t st) {
     if (!q || !k_layer || !v_layer || !meta || !scratch) return BONSAI_DECODE_ERR_ARG;
     if ((out_q == nullptr) != (out_s == nullptr)) return BONSAI_DECODE_ERR_ARG;
     if (!out_bf16 && !out_q) return BONSAI_DECODE_ERR_ARG;
@@ -1327,7 +1438,6 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
         n_heads > kCombineMaxHeads || sigma < 0 || sigma + M > slots ||
         (sigma + M + kChunk - 1) / kChunk > kCombineMaxChunks)
         return BONSAI_DECODE_ERR_ARG;
-    hipStream_t st = static_cast<hipStream_t>(stream);
     AttnArgs a;
     a.q = static_cast<const uint32_t *>(q);
     a.k_layer = static_cast<const uint32_t *>(k_layer);
@@ -1344,13 +1454,20 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
     // the live length is cache_len + M <= sigma + M: chunks beyond it are never launched
     a.n_chunks = (sigma + M + kChunk - 1) / kChunk;
     int parts = 0;  // partials per (row, head): chunks for the VALU pass, runs of chunks otherwise
-    if (g_attn_engine == 0) {
+    if (g_attn_engine == 0 || rope != nullptr) {
         parts = a.n_chunks < kMaxParts ? a.n_chunks : kMaxParts;
         const int tiles = (M * a.hpg + kPairTile - 1) / kPairTile;
-        hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_kv * parts * tiles), dim3(kAttnWaves * 64), 0, st,
-                           static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k_layer),
-                           static_cast<const uint16_t *>(v_layer), meta, a.part, a.scale_log2e, M,
-                           n_heads, n_kv, a.hpg, slots, sigma, parts);
+        const dim3 grid(n_kv * parts * tiles), block(kAttnWaves * 64);
+        if (rope != nullptr)
+            hipLaunchKernelGGL(attn_mfma_kernel<true>, grid, block, 0, st,
+                               static_cast<const uint16_t *>(q), static_cast<uint16_t *>(k_layer),
+                               static_cast<uint16_t *>(v_layer), meta, a.part, a.scale_log2e, M,
+                               n_heads, n_kv, a.hpg, slots, sigma, parts, *rope);
+        else
+            hipLaunchKernelGGL(attn_mfma_kernel<false>, grid, block, 0, st,
+                               static_cast<const uint16_t *>(q), static_cast<uint16_t *>(k_layer),
+                               static_cast<uint16_t *>(v_layer), meta, a.part, a.scale_log2e, M,
+                               n_heads, n_kv, a.hpg, slots, sigma, parts, RopeIn{});
     } else {
     const int rw = rows_per_wave(M);
     a.row_groups = (M + rw - 1) / rw;
@@ -1389,6 +1506,32 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
                            c.meta, c.out_bf16, c.out_q, c.out_s, c.M, c.n_heads, c.n_chunks,
                            c.sigma, c.parts);
     return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+}
+
+extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const void *v_layer,
+                                       const int32_t *meta, void *scratch, void *out_bf16,
+                                       int8_t *out_q, float *out_s, float scale, int M, int n_heads,
+                                       int n_kv, int slots, int sigma, void *stream) {
+    return launch_attention(q, const_cast<void *>(k_layer), const_cast<void *>(v_layer), meta, scratch,
+                            out_bf16, out_q, out_s, scale, M, n_heads, n_kv, slots, sigma, nullptr,
+                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int bonsai_decode_attention_rope(const void *xqkv, const void *q_norm_w, const void *k_norm_w,
+                                            float eps, const void *cos_table, const void *sin_table,
+                                            const int32_t *positions, int max_pos, void *k_layer,
+                                            void *v_layer, const int32_t *meta, void *scratch,
+                                            void *out_bf16, int8_t *out_q, float *out_s, float scale,
+                                            int M, int n_heads, int n_kv, int slots, int sigma,
+                                            void *stream) {
+    if (!q_norm_w || !k_norm_w || !cos_table || !sin_table || !positions || max_pos < 1)
+        return BONSAI_DECODE_ERR_ARG;
+    if (M > kRopeFusedMaxWidth) return BONSAI_DECODE_ERR_ARG;
+    const RopeIn rope{static_cast<const uint16_t *>(q_norm_w), static_cast<const uint16_t *>(k_norm_w),
+                      static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table),
+                      positions, eps, max_pos};
+    return launch_attention(xqkv, k_layer, v_layer, meta, scratch, out_bf16, out_q, out_s, scale, M,
+                            n_heads, n_kv, slots, sigma, &rope, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int bonsai_kv_commit(void *kv, int n_layers, int n_kv, int slots, int src_slot,

@@ -15,6 +15,7 @@ iteration); the forced run commits whole blocks.  Prompt ids are uniform random.
 from __future__ import annotations
 
 import argparse
+import os
 import json
 import time
 
@@ -127,10 +128,13 @@ def run_slot_costs(model_name: str = "1.7b", cache_len: int = 500, device: str =
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / replays * 1e3
 
-    saved = (mdl._gemv, decode_ops.qk_norm_rope_kv_write, decode_ops.decode_attention, ops.actq_lib)
+    saved = (mdl._gemv, decode_ops.qk_norm_rope_kv_write, decode_ops.decode_attention, ops.actq_lib,
+             mdl._fused, os.environ.get("BONSAI_FUSED_STEP"))
     out = {"model": model_name, "cache_len": cache_len, "widths": {}}
     try:
         for M, role in ((1, "ar"), (9, "verify")):
+            # the ten-launch layer (what widths above two always run)
+            os.environ["BONSAI_FUSED_STEP"] = "0"
             base = graph_us(M, role)
             row = {"graph_us": round(base, 1), "launches": 10 * n_layers + 4}
             mdl._gemv = lambda *a, **k: None
@@ -148,9 +152,31 @@ def run_slot_costs(model_name: str = "1.7b", cache_len: int = 500, device: str =
                                                        "bonsai_rmsnorm_quant_int8"})
             row["add_norm_quant_us_per_launch"] = round((base - graph_us(M, role)) / (2 * n_layers + 1), 2)
             ops.actq_lib = saved[3]
+            if M <= ops.FUSED_MAX_TOKENS:
+                # the seven-launch layer: each fused projection by what it reads and stores
+                os.environ["BONSAI_FUSED_STEP"] = "1"
+                fbase = graph_us(M, role)
+                frow = {"graph_us": round(fbase, 1), "launches": 7 * n_layers + 5}
+                for label, act_kind, epi in (("qkv_norm_in", ops.ACT_BF16_NORM, ops.EPI_PLAIN),
+                                             ("o_add_out", ops.ACT_INT8, ops.EPI_ADD_SUMSQ),
+                                             ("gate_up_norm_in_silu_out", ops.ACT_BF16_NORM, ops.EPI_SILU_PAIR),
+                                             ("down_amax_in_add_out", ops.ACT_BF16_AMAX, ops.EPI_ADD_SUMSQ)):
+                    def without(w, m, stream, _skip=(act_kind, epi), **kw):
+                        if (kw["act_kind"], kw["epi"]) != _skip:
+                            saved[4](w, m, stream, **kw)
+                    mdl._fused = without
+                    n = n_layers - 1 if label == "qkv_norm_in" else n_layers
+                    frow[label + "_us_per_launch"] = round((fbase - graph_us(M, role)) / n, 2)
+                    mdl._fused = saved[4]
+                row["fused_layers"] = frow
             out["widths"][str(M)] = row
     finally:
-        mdl._gemv, decode_ops.qk_norm_rope_kv_write, decode_ops.decode_attention, ops.actq_lib = saved
+        (mdl._gemv, decode_ops.qk_norm_rope_kv_write, decode_ops.decode_attention, ops.actq_lib,
+         mdl._fused) = saved[:5]
+        if saved[5] is None:
+            os.environ.pop("BONSAI_FUSED_STEP", None)
+        else:
+            os.environ["BONSAI_FUSED_STEP"] = saved[5]
     return out
 
 

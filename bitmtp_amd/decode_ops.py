@@ -42,6 +42,9 @@ def load_decode_kernel() -> None:
     lib.bonsai_decode_attention.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, cf,
                                             ci, ci, ci, ci, ci, vp]
     lib.bonsai_decode_attention.restype = ci
+    lib.bonsai_decode_attention_rope.argtypes = [vp, vp, vp, cf, vp, vp, vp, ci, vp, vp, vp, vp, vp, vp, vp,
+                                                 cf, ci, ci, ci, ci, ci, vp]
+    lib.bonsai_decode_attention_rope.restype = ci
     lib.bonsai_decode_set_tuning.argtypes = [ci]
     lib.bonsai_decode_set_tuning.restype = None
     lib.bonsai_decode_set_attention_engine.argtypes = [ci]
@@ -163,6 +166,57 @@ def decode_attention(q: torch.Tensor, k_layer: torch.Tensor, v_layer: torch.Tens
             _ptr(out_q), _ptr(out_s), float(scale), m, n_heads, n_kv, slots, int(sigma),
             _stream(q.device))
     _need(rc == 0, f"bonsai_decode_attention failed with status {rc}")
+
+
+ROPE_FUSED_MAX_WIDTH = 2
+
+
+def decode_attention_rope(xqkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: torch.Tensor, eps: float,
+                          cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                          k_layer: torch.Tensor, v_layer: torch.Tensor, meta: torch.Tensor,
+                          scratch: torch.Tensor, sigma: int, n_heads: int,
+                          out_bf16: Optional[torch.Tensor] = None, out_q: Optional[torch.Tensor] = None,
+                          out_s: Optional[torch.Tensor] = None, scale: Optional[float] = None) -> None:
+    """:func:`qk_norm_rope_kv_write` and :func:`decode_attention` in two launches instead of three,
+    for blocks of one or two rows: the attention derives q and the block's own K / V rows from the
+    merged projection ``xqkv`` itself (same bits) and writes the K / V rows to slots ``sigma ..``
+    (reference: model.py:388-436 and :996-1005)."""
+    m = xqkv.shape[0]
+    n_kv, slots = k_layer.shape[0], k_layer.shape[1]
+    for t, name in ((xqkv, "xqkv"), (q_norm_w, "q_norm_w"), (k_norm_w, "k_norm_w"), (cos, "cos"),
+                    (sin, "sin"), (k_layer, "k_layer"), (v_layer, "v_layer")):
+        _check(t, torch.bfloat16, name)
+    _check(positions, torch.int32, "positions")
+    _check(meta, torch.int32, "meta")
+    _need(m <= ROPE_FUSED_MAX_WIDTH, "at most two rows: use qk_norm_rope_kv_write + decode_attention")
+    _need(xqkv.shape == (m, (n_heads + 2 * n_kv) * HEAD_DIM), "xqkv shape mismatch")
+    _need(k_layer.shape == v_layer.shape and k_layer.dim() == 3 and k_layer.shape[2] == HEAD_DIM,
+          "KV layer shape mismatch")
+    _need(cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == HEAD_DIM,
+          "RoPE table shape mismatch")
+    _need(positions.numel() == m and q_norm_w.numel() == HEAD_DIM and k_norm_w.numel() == HEAD_DIM,
+          "positions / norm weight size mismatch")
+    _need(meta.numel() >= 2 + m, "meta needs 2 + M entries")
+    _need(scratch.is_cuda and scratch.is_contiguous()
+          and scratch.numel() * scratch.element_size() >= attention_scratch_bytes(m, n_heads, slots),
+          "attention scratch too small")
+    if out_bf16 is not None:
+        _check(out_bf16, torch.bfloat16, "out_bf16")
+        _need(out_bf16.numel() == m * n_heads * HEAD_DIM, "out_bf16 size mismatch")
+    if out_q is not None or out_s is not None:
+        _need(out_q is not None and out_s is not None, "out_q and out_s come together")
+        _check(out_q, torch.int8, "out_q")
+        _check(out_s, torch.float32, "out_s")
+        _need(out_q.numel() == m * n_heads * HEAD_DIM and out_s.numel() == m, "out_q/out_s size mismatch")
+    if scale is None:
+        scale = 1.0 / math.sqrt(HEAD_DIM)
+    with torch.cuda.device(xqkv.device):
+        rc = decode_lib().bonsai_decode_attention_rope(
+            _ptr(xqkv), _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(cos), _ptr(sin), _ptr(positions),
+            cos.shape[0], _ptr(k_layer), _ptr(v_layer), _ptr(meta), _ptr(scratch), _ptr(out_bf16),
+            _ptr(out_q), _ptr(out_s), float(scale), m, n_heads, n_kv, slots, int(sigma),
+            _stream(xqkv.device))
+    _need(rc == 0, f"bonsai_decode_attention_rope failed with status {rc}")
 
 
 def kv_commit(kv: torch.Tensor, src_slot: int, dst_slot: int, n: int) -> None:

@@ -461,8 +461,8 @@ class FusedPlan:
 
 def fused_plan(model: "BonsaiDecoder", m: int) -> Optional[FusedPlan]:
     """How a step of width ``m`` runs its layers: with the residual add + RMSNorm + quantisation
-    and the SiLU * up + quantisation folded into the projections (seven launches a layer instead of
-    ten; blocks of one or two tokens), or -- ``None`` -- with the separate producers (wider blocks,
+    and the SiLU * up + quantisation folded into the projections and q / k norm + RoPE into the attention (six
+    launches a layer instead of ten; blocks of one or two tokens), or -- ``None`` -- with the separate producers (wider blocks,
     shapes the fused kernels do not take, BONSAI_FUSED_STEP=0)."""
     if m > ops.FUSED_MAX_TOKENS or os.environ.get("BONSAI_FUSED_STEP", "1") == "0":
         return None
@@ -525,7 +525,8 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
     torch.index_select(model.embed, 0, io.tokens, out=h_cur)
     for i, lw in enumerate(model.layers):
         if plan is not None:
-            # seven launches: the element-wise producers ride in the projections on either side;
+            # six launches: the element-wise producers ride in the projections on either side and
+            # the q / k norm + RoPE in the attention;
             # h_cur already holds the residual stream including the previous layer's MLP
             if i == 0:
                 check(actq.bonsai_rmsnorm_quant_int8(_vp(h_cur), _vp(lw.input_layernorm), eps,
@@ -536,11 +537,10 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
                 _fused(lw.wqkv, M, stream, act=h_cur, act_aux=ws.sumsq, act_kind=ops.ACT_BF16_NORM,
                        act_parts=plan.down, norm_w=lw.input_layernorm, eps=eps, out=ws.xqkv,
                        epi=ops.EPI_PLAIN)
-            decode_ops.qk_norm_rope_kv_write(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
-                                             io.positions, ws.q[:M], kv[0, i], kv[1, i],
-                                             args.n_heads, args.n_kv_heads, sigma)
-            decode_ops.decode_attention(ws.q[:M], kv[0, i], kv[1, i], io.meta, ws.attn_scratch, sigma,
-                                        out_q=ws.o_q[:M], out_s=ws.o_s[:M])
+            decode_ops.decode_attention_rope(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
+                                             io.positions, kv[0, i], kv[1, i], io.meta,
+                                             ws.attn_scratch, sigma, args.n_heads,
+                                             out_q=ws.o_q[:M], out_s=ws.o_s[:M])
             _fused(lw.wo, M, stream, act=ws.o_q, act_aux=ws.o_s, act_kind=ops.ACT_INT8, out=h_nxt,
                    epi=ops.EPI_ADD_SUMSQ, residual=h_cur, out_aux=ws.sumsq)
             h_cur, h_nxt = h_nxt, h_cur

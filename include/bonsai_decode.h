@@ -93,6 +93,22 @@ int bonsai_decode_attention(const void *q, const void *k_layer, const void *v_la
                             float *out_s, float scale, int M, int n_heads, int n_kv, int slots,
                             int sigma, void *stream);
 
+/* bonsai_qk_norm_rope_kv_write and bonsai_decode_attention as one call (two launches instead of
+ * three) for blocks of one or two rows: the chunk pass of the attention derives its q rows and
+ * the block's own K / V rows from the merged projection itself, with the arithmetic and rounding
+ * points stated for bonsai_qk_norm_rope_kv_write (same bits), uses them without a round trip
+ * through the cache, and writes the K / V rows to slots sigma .. sigma + M - 1 for later steps.
+ * No counterpart in the reference beyond the two functions this stands for (model.py:388-436
+ * and :996-1004); a one-token decode step spends as long on the separate RoPE launch as on the
+ * attention itself.  Operands as for those two functions; always the matrix-core chunk pass;
+ * M <= 2 (BONSAI_DECODE_ERR_ARG otherwise: use the two calls). */
+int bonsai_decode_attention_rope(const void *xqkv, const void *q_norm_w, const void *k_norm_w,
+                                 float eps, const void *cos_table, const void *sin_table,
+                                 const int32_t *positions, int max_pos, void *k_layer, void *v_layer,
+                                 const int32_t *meta, void *scratch, void *out_bf16, int8_t *out_q,
+                                 float *out_s, float scale, int M, int n_heads, int n_kv, int slots,
+                                 int sigma, void *stream);
+
 /* Copies n KV rows of every layer and kv head from slot src to slot dst inside one
  * shared buffer [2, n_layers, n_kv, slots, 128] bf16 (commit_kv / commit_kv_from_verify,
  * src/bonsai_sft/gpu/fast_runtime.py:467-508).  Source and destination ranges must

@@ -320,6 +320,81 @@ def test_argument_checks():
         ops.packed_gemv_fused(inner, w_dn.weight, w_dn.weight_scale, bits=bits, amax=amax, s=x_s, parts=parts)
 
 
+ROPE_CASES = [
+    # M, n_heads, n_kv, sigma, cache_len, role
+    (1, 16, 8, 1024, 500, "ar"),
+    (1, 16, 8, 1024, 0, "ar"),        # nothing but the row itself
+    (1, 16, 8, 1024, 63, "ar"),       # the row is the last slot of a chunk
+    (1, 16, 8, 1024, 64, "ar"),       # ... the first slot of the next
+    (2, 16, 8, 1024, 63, "ar"),       # the two rows sit in two chunks (and two workgroups)
+    (2, 32, 8, 4096, 1531, "ar"),     # four query heads per kv head
+    (1, 32, 8, 4096, 4095, "ar"),
+    (2, 4, 2, 256, 255, "verify"),
+    (1, 6, 2, 64, 17, "ar"),
+]
+
+
+@pytest.mark.parametrize("M,n_heads,n_kv,sigma,cache_len,role", ROPE_CASES)
+def test_attention_with_rope_inside_gives_the_bits_of_the_two_calls(M, n_heads, n_kv, sigma, cache_len, role):
+    """bonsai_decode_attention_rope against bonsai_qk_norm_rope_kv_write + bonsai_decode_attention:
+    the bf16 and the quantised attention output and the K / V rows it leaves in the cache are the
+    same bits; no other cache row is touched."""
+    from bitmtp_amd import decode_ops, runtime
+    print(f"[case] attention with rope inside M={M} heads={n_heads}/{n_kv} sigma={sigma} "
+          f"cache_len={cache_len} {role}", flush=True)
+    gen = _gen(M + n_heads + sigma + cache_len)
+    slots = sigma + 17
+    hd = 128
+    xqkv = _rows(gen, M, (n_heads + 2 * n_kv) * hd, 1.5)
+    qw = (1.0 + 0.1 * torch.randn(hd, generator=gen, device=DEV)).to(torch.bfloat16)
+    kw = (1.0 + 0.1 * torch.randn(hd, generator=gen, device=DEV)).to(torch.bfloat16)
+    max_pos = 8192
+    ang = torch.rand(max_pos, hd, generator=gen, device=DEV) * 6.28
+    cos, sin = torch.cos(ang).to(torch.bfloat16), torch.sin(ang).to(torch.bfloat16)
+    positions = torch.tensor([cache_len + i for i in range(M)], dtype=torch.int32, device=DEV)
+    kv0 = (torch.randn(2, n_kv, slots, hd, generator=gen, device=DEV) * 1.2).to(torch.bfloat16)
+    meta = torch.tensor(runtime.step_descriptor(role, M, 8, cache_len, 0), dtype=torch.int32, device=DEV)
+    scratch = torch.empty(decode_ops.attention_scratch_bytes(M, n_heads, slots) // 4, dtype=torch.float32,
+                          device=DEV)
+
+    def outs():
+        return (torch.zeros(M, n_heads * hd, dtype=torch.bfloat16, device=DEV),
+                torch.zeros(M, n_heads * hd, dtype=torch.int8, device=DEV),
+                torch.zeros(M, dtype=torch.float32, device=DEV))
+
+    kv_a = kv0.clone()
+    q = torch.empty(M, n_heads, hd, dtype=torch.bfloat16, device=DEV)
+    decode_ops.qk_norm_rope_kv_write(xqkv, qw, kw, EPS, cos, sin, positions, q, kv_a[0], kv_a[1], n_heads,
+                                     n_kv, sigma)
+    o_a, q_a, s_a = outs()
+    decode_ops.decode_attention(q, kv_a[0], kv_a[1], meta, scratch, sigma, out_bf16=o_a, out_q=q_a, out_s=s_a)
+    torch.cuda.synchronize()
+
+    kv_b = kv0.clone()
+    o_b, q_b, s_b = outs()
+    scratch.fill_(float("nan"))
+    decode_ops.decode_attention_rope(xqkv, qw, kw, EPS, cos, sin, positions, kv_b[0], kv_b[1], meta, scratch,
+                                     sigma, n_heads, out_bf16=o_b, out_q=q_b, out_s=s_b)
+    torch.cuda.synchronize()
+    assert _same_bits(o_a, o_b) and torch.equal(q_a, q_b) and torch.equal(s_a, s_b)
+    assert torch.equal(kv_a.view(torch.int16), kv_b.view(torch.int16))
+    changed = (kv_b.view(torch.int16) != kv0.view(torch.int16)).any(dim=-1)   # [2, n_kv, slots]
+    assert not changed[:, :, :sigma].any() and not changed[:, :, sigma + M:].any()
+
+
+def test_attention_with_rope_inside_refuses_wide_blocks():
+    from bitmtp_amd import decode_ops
+    xqkv = torch.zeros(3, (4 + 4) * 128, dtype=torch.bfloat16, device=DEV)
+    w = torch.ones(128, dtype=torch.bfloat16, device=DEV)
+    tab = torch.ones(16, 128, dtype=torch.bfloat16, device=DEV)
+    kv = torch.zeros(2, 2, 80, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        decode_ops.decode_attention_rope(xqkv, w, w, EPS, tab, tab, torch.zeros(3, dtype=torch.int32, device=DEV),
+                                         kv[0], kv[1], torch.zeros(5, dtype=torch.int32, device=DEV),
+                                         torch.zeros(1 << 16, dtype=torch.float32, device=DEV), 64, 4,
+                                         out_bf16=torch.zeros(3, 512, dtype=torch.bfloat16, device=DEV))
+
+
 @pytest.mark.parametrize("kind", ["t2g128", "q1"])
 def test_decode_loop_tokens_do_not_depend_on_the_fused_layers(kind, monkeypatch):
     """Greedy AR decoding (width-1 steps) through graphs captured with and without the fused
