@@ -424,7 +424,9 @@ __device__ __forceinline__ void gemv_dot4_body(const GemvArgs &a, int bx, int by
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int idx = lane + 64 * j;
-                part_raw[m][j] = prow[idx < a.in_count ? idx : 0];  // past the end: not added below
+                part_raw[m][j] = 0.0;
+                if (64 * j < a.in_count)  // uniform: no load for a run of 64 parts that does not exist
+                    part_raw[m][j] = prow[idx < a.in_count ? idx : 0];  // past the end: not added below
             }
         }
     }

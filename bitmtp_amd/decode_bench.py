@@ -153,10 +153,15 @@ def run_slot_costs(model_name: str = "1.7b", cache_len: int = 500, device: str =
             row["add_norm_quant_us_per_launch"] = round((base - graph_us(M, role)) / (2 * n_layers + 1), 2)
             ops.actq_lib = saved[3]
             if M <= ops.FUSED_MAX_TOKENS:
-                # the seven-launch layer: each fused projection by what it reads and stores
+                # the six-launch layer: each fused projection by what it reads and stores, and the
+                # attention that derives q / k itself (two launches)
                 os.environ["BONSAI_FUSED_STEP"] = "1"
                 fbase = graph_us(M, role)
-                frow = {"graph_us": round(fbase, 1), "launches": 7 * n_layers + 5}
+                frow = {"graph_us": round(fbase, 1), "launches": 6 * n_layers + 5}
+                rope_attn = decode_ops.decode_attention_rope
+                decode_ops.decode_attention_rope = lambda *a, **k: None
+                frow["attention_with_rope_us_per_layer_2_launches"] = round((fbase - graph_us(M, role)) / n_layers, 2)
+                decode_ops.decode_attention_rope = rope_attn
                 for label, act_kind, epi in (("qkv_norm_in", ops.ACT_BF16_NORM, ops.EPI_PLAIN),
                                              ("o_add_out", ops.ACT_INT8, ops.EPI_ADD_SUMSQ),
                                              ("gate_up_norm_in_silu_out", ops.ACT_BF16_NORM, ops.EPI_SILU_PAIR),
