@@ -429,13 +429,14 @@ int launch_gemv(const int8_t *A, const uint8_t *B, void *out, const float *s, co
 constexpr int kFusedMaxWidth = kFusedMaxTile;
 
 template <int BITS>
-int fused_ready(int M, int N, int K, hipStream_t stream, int *lds_limit) {
+int fused_ready(int M, int N, int K, hipStream_t stream, int *lds_limit, int *n_cus) {
     if (M < 1 || M > kFusedMaxWidth || N < 1 || K < kGroup || K % kGroup != 0) return 1;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 2;
     const int rc = ensure_ready<BITS>(dev, stream);
     if (rc != 0) return rc;
     *lds_limit = lib_state<BITS>().lds_limit[dev];
+    *n_cus = lib_state<BITS>().n_cus[dev];
     return 0;
 }
 
@@ -445,10 +446,10 @@ template <int BITS>
 int fused_parts(int epi, int M, int N, int K) {
     if (epi != EPI_SILU_PAIR && epi != EPI_ADD_SUMSQ) return -1;
     if (epi == EPI_SILU_PAIR && (N < 2 || (N & 1))) return -1;
-    int lds_limit = 0;
-    const int rc = fused_ready<BITS>(M, N, K, nullptr, &lds_limit);
+    int lds_limit = 0, n_cus = 0;
+    const int rc = fused_ready<BITS>(M, N, K, nullptr, &lds_limit, &n_cus);
     if (rc != 0) return -rc;
-    const Geometry g = fused_geometry<BITS>(epi, M, N, K, lds_limit);
+    const Geometry g = fused_geometry<BITS>(PRO_INT8, epi, M, N, K, lds_limit, n_cus);
     return g.mt == 0 ? -1 : g.grid_x;
 }
 
@@ -476,10 +477,10 @@ int launch_gemv_fused(const FusedGemv &d, hipStream_t stream) {
         if (d.epi == EPI_SILU_PAIR && (d.N < 2 || (d.N & 1) || mis(d.out_aux, 16))) return 1;
         if (d.epi == EPI_ADD_SUMSQ && (d.residual == nullptr || mis(d.residual, 2) || mis(d.out_aux, 8))) return 1;
     }
-    int lds_limit = 0;
-    const int rc = fused_ready<BITS>(d.M, d.N, d.K, stream, &lds_limit);
+    int lds_limit = 0, n_cus = 0;
+    const int rc = fused_ready<BITS>(d.M, d.N, d.K, stream, &lds_limit, &n_cus);
     if (rc != 0) return rc;
-    return launch_gemv_dot4_fused<BITS>(d, lds_limit, stream);
+    return launch_gemv_dot4_fused<BITS>(d, lds_limit, n_cus, stream);
 }
 
 // Several GEMVs in one call (descriptors in host memory, read before the call returns).
