@@ -108,8 +108,11 @@ def test_mlp_tail_two_launches_give_the_bits_of_three(dot4_only, bits, M, dim, f
         assert _same_bits(got, ref), f"out_kind {kind}"
 
 
+# (5120 and 8192 columns at two tokens: more quarters than a workgroup has threads, so the staging
+# loops past each thread's first quarter run too)
 @pytest.mark.parametrize("n_prod,k_prod,n_cons", [(2048, 2048, 4096), (2048, 6144, 12288), (2560, 9728, 6144),
-                                                  (512, 512, 1024), (384, 1408, 256), (128, 128, 128)])
+                                                  (512, 512, 1024), (384, 1408, 256), (128, 128, 128),
+                                                  (5120, 1024, 640), (8192, 512, 20480)])
 @pytest.mark.parametrize("M", [1, 2])
 @pytest.mark.parametrize("bits", [2, 1])
 def test_add_norm_quant_rides_in_the_projections(dot4_only, bits, M, n_prod, k_prod, n_cons):
