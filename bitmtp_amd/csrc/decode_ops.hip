@@ -78,21 +78,32 @@ struct RopeArgs {
 
 // RMSNorm + RoPE of one 128-wide head row by one wave: lane i holds the pair (i, i + 64) in
 // (r0, r1) and receives the finished pair in (o0b, o1b) as bf16 bits.
-__device__ __forceinline__ void qk_norm_rope_row(uint32_t r0, uint32_t r1, const uint16_t *w,
-                                                 const uint16_t *cos_t, const uint16_t *sin_t, int pos,
-                                                 int max_pos, float eps, int lane, uint32_t &o0b,
-                                                 uint32_t &o1b) {
-    const float f0 = bf16_bits_to_f32(r0), f1 = bf16_bits_to_f32(r1);
-    const double ss = bonsai_wave::sum64((double)(f0 * f0) + (double)(f1 * f1));
-    const float var = (float)ss / (float)kHd;
-    const float rs = 1.0f / sqrtf(var + eps);
-    const float n0 = bf16_round(bf16_bits_to_f32(w[lane]) * bf16_round(f0 * rs));
-    const float n1 = bf16_round(bf16_bits_to_f32(w[lane + 64]) * bf16_round(f1 * rs));
+// What a lane holds of one such row (bf16 bits): the pair, its norm weights, the cos / sin entries
+// of the row's position.  Loading and arithmetic are apart so that a wave can have several rows'
+// loads in flight.
+struct RopeRowIn {
+    uint32_t r0, r1, w0, w1, c0, c1, s0, s1;
+};
+
+__device__ __forceinline__ RopeRowIn rope_row_load(const uint16_t *x, const uint16_t *w,
+                                                   const uint16_t *cos_t, const uint16_t *sin_t, int pos,
+                                                   int max_pos, int lane) {
     pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
     const uint16_t *cr = cos_t + (size_t)pos * kHd;
     const uint16_t *sr = sin_t + (size_t)pos * kHd;
-    const float c0 = bf16_bits_to_f32(cr[lane]), c1 = bf16_bits_to_f32(cr[lane + 64]);
-    const float s0 = bf16_bits_to_f32(sr[lane]), s1 = bf16_bits_to_f32(sr[lane + 64]);
+    return RopeRowIn{x[lane], x[lane + 64], w[lane], w[lane + 64], cr[lane], cr[lane + 64], sr[lane],
+                     sr[lane + 64]};
+}
+
+__device__ __forceinline__ void rope_row_math(const RopeRowIn &in, float eps, uint32_t &o0b, uint32_t &o1b) {
+    const float f0 = bf16_bits_to_f32(in.r0), f1 = bf16_bits_to_f32(in.r1);
+    const double ss = bonsai_wave::sum64((double)(f0 * f0) + (double)(f1 * f1));
+    const float var = (float)ss / (float)kHd;
+    const float rs = 1.0f / sqrtf(var + eps);
+    const float n0 = bf16_round(bf16_bits_to_f32(in.w0) * bf16_round(f0 * rs));
+    const float n1 = bf16_round(bf16_bits_to_f32(in.w1) * bf16_round(f1 * rs));
+    const float c0 = bf16_bits_to_f32(in.c0), c1 = bf16_bits_to_f32(in.c1);
+    const float s0 = bf16_bits_to_f32(in.s0), s1 = bf16_bits_to_f32(in.s1);
     // rotate_half(n) = [-n_hi, n_lo]
     const float o0 = bf16_round(bf16_round(n0 * c0) + bf16_round(-n1 * s0));
     const float o1 = bf16_round(bf16_round(n1 * c1) + bf16_round(n0 * s1));
@@ -125,8 +136,8 @@ qk_norm_rope_kernel(const uint16_t *pxqkv, const uint16_t *pqw, const uint16_t *
     }
     const bool is_q = head < a.n_heads;
     uint32_t o0, o1;
-    qk_norm_rope_row(r0, r1, is_q ? a.qw : a.kw, a.cos_t, a.sin_t, a.positions[m], a.max_pos, a.eps,
-                     lane, o0, o1);
+    rope_row_math(rope_row_load(x, is_q ? a.qw : a.kw, a.cos_t, a.sin_t, a.positions[m], a.max_pos, lane),
+                  a.eps, o0, o1);
     uint16_t *dst = is_q ? a.q_out + ((size_t)m * a.n_heads + head) * kHd
                          : a.k_layer + ((size_t)(head - a.n_heads) * a.slots + a.write_slot + m) * kHd;
     dst[lane] = (uint16_t)o0;
@@ -313,15 +324,12 @@ __host__ __device__ inline int attn_chunks_per_part(int live_chunks, int parts) 
 }
 
 // ROPE: the launch takes the merged q|k|v projection instead of finished q rows and does the work
-// of qk_norm_rope_kernel itself, for blocks of at most kRopeFusedMaxWidth tokens (a decode step
-// of one token spends as long on that launch as on this one).  Every workgroup derives the q rows
-// of its pair tile -- one wave per (token, head) row, the very arithmetic of qk_norm_rope_kernel --
+// of qk_norm_rope_kernel itself (a decode step of one token spends as long on that launch as on
+// this one).  Every workgroup derives the q rows of its pair tile -- one wave per (token, head) row, the very arithmetic of qk_norm_rope_kernel --
 // and hands them to its waves through LDS; a workgroup whose chunks reach the block's own rows
 // (logical index >= cache_len) derives those K rows the same way and takes the V rows from the
 // projection, never from the cache, so no workgroup uses what another one writes; the workgroup
 // of pair tile 0 that owns a row's chunk also writes it to the cache for the steps to come.
-constexpr int kRopeFusedMaxWidth = 2;
-
 struct RopeIn {
     const uint16_t *qw, *kw, *cos_t, *sin_t;
     const int32_t *positions;
@@ -336,8 +344,8 @@ attn_mfma_kernel(const uint16_t *q, uint16_t *k_layer, uint16_t *v_layer,
                  int n_kv, int G, int slots, int sigma, int parts, const RopeIn rope) {
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kChunk * kVPitch];
     __shared__ __attribute__((aligned(16))) uint16_t q_new[ROPE ? kPairTile : 1][kHd];
-    __shared__ __attribute__((aligned(16))) uint16_t k_new[ROPE ? kRopeFusedMaxWidth : 1][kHd];
-    __shared__ __attribute__((aligned(16))) uint16_t v_new[ROPE ? kRopeFusedMaxWidth : 1][kHd];
+    __shared__ __attribute__((aligned(16))) uint16_t k_new[ROPE ? BONSAI_MAX_WIDTH : 1][kHd];
+    __shared__ __attribute__((aligned(16))) uint16_t v_new[ROPE ? BONSAI_MAX_WIDTH : 1][kHd];
     __shared__ __attribute__((aligned(16))) unsigned char p_lds[kPairTile * kPPitch];
     __shared__ __attribute__((aligned(16))) float st_max[kAttnWaves][kPairTile];
     __shared__ __attribute__((aligned(16))) float st_sum[kAttnWaves][kPairTile];
@@ -450,38 +458,52 @@ attn_mfma_kernel(const uint16_t *q, uint16_t *k_layer, uint16_t *v_layer,
         const int total_heads = n_heads + 2 * n_kv;
         const int n_q = min(kPairTile, pairs_total - pt * kPairTile);
         const int n_jobs = n_q + (own_rows ? M : 0);
-        for (int job = w; job < n_jobs; job += kAttnWaves) {
-            const bool is_q = job < n_q;
-            int m, src_head;
-            if (is_q) {
+        // a job is one row: q row `job` of the tile, then K row (with its V row) job - n_q of the
+        // block.  A wave takes kRowsInFlight jobs at a time and issues all their loads first.
+        constexpr int kRowsInFlight = 4;
+        const int wu = __builtin_amdgcn_readfirstlane(w);
+        for (int base = 0; base < n_jobs; base += kRowsInFlight * kAttnWaves) {
+            RopeRowIn in[kRowsInFlight];
+            uint16_t v0[kRowsInFlight], v1[kRowsInFlight];
+            int jm[kRowsInFlight];
+#pragma unroll
+            for (int j = 0; j < kRowsInFlight; ++j) {
+                const int job = min(base + wu + j * kAttnWaves, n_jobs - 1);  // past the end: a repeat, unused
+                const bool is_q = job < n_q;
                 const int qp = pt * kPairTile + job;
-                m = qp / G;
-                src_head = kvh * G + (qp - m * G);
-            } else {
-                m = job - n_q;
-                src_head = n_heads + kvh;
+                jm[j] = is_q ? qp / G : job - n_q;
+                const int src_head = is_q ? kvh * G + (qp - jm[j] * G) : n_heads + kvh;
+                in[j] = rope_row_load(q + ((size_t)jm[j] * total_heads + src_head) * kHd,
+                                      is_q ? rope.qw : rope.kw, rope.cos_t, rope.sin_t,
+                                      rope.positions[jm[j]], rope.max_pos, lane);
+                const uint16_t *xv = q + ((size_t)jm[j] * total_heads + n_heads + n_kv + kvh) * kHd;
+                v0[j] = xv[lane];
+                v1[j] = xv[lane + 64];
             }
-            const uint16_t *x = q + ((size_t)m * total_heads + src_head) * kHd;
-            uint32_t o0, o1;
-            qk_norm_rope_row(x[lane], x[lane + 64], is_q ? rope.qw : rope.kw, rope.cos_t, rope.sin_t,
-                             rope.positions[m], rope.max_pos, rope.eps, lane, o0, o1);
-            uint16_t *dst = is_q ? q_new[job] : k_new[m];
-            dst[lane] = (uint16_t)o0;
-            dst[lane + 64] = (uint16_t)o1;
-            if (!is_q) {
-                const uint16_t *xv = q + ((size_t)m * total_heads + n_heads + n_kv + kvh) * kHd;
-                const uint16_t v0 = xv[lane], v1 = xv[lane + 64];
-                v_new[m][lane] = v0;
-                v_new[m][lane + 64] = v1;
-                // the cache row, once: by the workgroup of pair tile 0 that owns the row's chunk
-                const int c_row = (cache_len + m) / kChunk;
-                if (pt == 0 && c_row >= c_begin && c_row < c_end) {
-                    uint16_t *kd = k_layer + ((size_t)kvh * slots + sigma + m) * kHd;
-                    uint16_t *vd = v_layer + ((size_t)kvh * slots + sigma + m) * kHd;
-                    kd[lane] = (uint16_t)o0;
-                    kd[lane + 64] = (uint16_t)o1;
-                    vd[lane] = v0;
-                    vd[lane + 64] = v1;
+#pragma unroll
+            for (int j = 0; j < kRowsInFlight; ++j) {
+                const int job = base + wu + j * kAttnWaves;
+                if (job >= n_jobs) break;  // uniform
+                const bool is_q = job < n_q;
+                const int m = jm[j];
+                uint32_t o0, o1;
+                rope_row_math(in[j], rope.eps, o0, o1);
+                uint16_t *dst = is_q ? q_new[job] : k_new[m];
+                dst[lane] = (uint16_t)o0;
+                dst[lane + 64] = (uint16_t)o1;
+                if (!is_q) {
+                    v_new[m][lane] = v0[j];
+                    v_new[m][lane + 64] = v1[j];
+                    // the cache row, once: by the workgroup of pair tile 0 that owns the row's chunk
+                    const int c_row = (cache_len + m) / kChunk;
+                    if (pt == 0 && c_row >= c_begin && c_row < c_end) {
+                        uint16_t *kd = k_layer + ((size_t)kvh * slots + sigma + m) * kHd;
+                        uint16_t *vd = v_layer + ((size_t)kvh * slots + sigma + m) * kHd;
+                        kd[lane] = (uint16_t)o0;
+                        kd[lane + 64] = (uint16_t)o1;
+                        vd[lane] = v0[j];
+                        vd[lane + 64] = v1[j];
+                    }
                 }
             }
         }
@@ -1526,7 +1548,6 @@ extern "C" int bonsai_decode_attention_rope(const void *xqkv, const void *q_norm
                                             void *stream) {
     if (!q_norm_w || !k_norm_w || !cos_table || !sin_table || !positions || max_pos < 1)
         return BONSAI_DECODE_ERR_ARG;
-    if (M > kRopeFusedMaxWidth) return BONSAI_DECODE_ERR_ARG;
     const RopeIn rope{static_cast<const uint16_t *>(q_norm_w), static_cast<const uint16_t *>(k_norm_w),
                       static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table),
                       positions, eps, max_pos};

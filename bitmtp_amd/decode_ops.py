@@ -168,7 +168,7 @@ def decode_attention(q: torch.Tensor, k_layer: torch.Tensor, v_layer: torch.Tens
     _need(rc == 0, f"bonsai_decode_attention failed with status {rc}")
 
 
-ROPE_FUSED_MAX_WIDTH = 2
+ROPE_FUSED_MAX_WIDTH = MAX_WIDTH
 
 
 def decode_attention_rope(xqkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: torch.Tensor, eps: float,
@@ -178,7 +178,7 @@ def decode_attention_rope(xqkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: 
                           out_bf16: Optional[torch.Tensor] = None, out_q: Optional[torch.Tensor] = None,
                           out_s: Optional[torch.Tensor] = None, scale: Optional[float] = None) -> None:
     """:func:`qk_norm_rope_kv_write` and :func:`decode_attention` in two launches instead of three,
-    for blocks of one or two rows: the attention derives q and the block's own K / V rows from the
+    the attention derives q and the block's own K / V rows from the
     merged projection ``xqkv`` itself (same bits) and writes the K / V rows to slots ``sigma ..``
     (reference: model.py:388-436 and :996-1005)."""
     m = xqkv.shape[0]
@@ -188,7 +188,7 @@ def decode_attention_rope(xqkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: 
         _check(t, torch.bfloat16, name)
     _check(positions, torch.int32, "positions")
     _check(meta, torch.int32, "meta")
-    _need(m <= ROPE_FUSED_MAX_WIDTH, "at most two rows: use qk_norm_rope_kv_write + decode_attention")
+    _need(1 <= m <= ROPE_FUSED_MAX_WIDTH, f"1..{ROPE_FUSED_MAX_WIDTH} rows")
     _need(xqkv.shape == (m, (n_heads + 2 * n_kv) * HEAD_DIM), "xqkv shape mismatch")
     _need(k_layer.shape == v_layer.shape and k_layer.dim() == 3 and k_layer.shape[2] == HEAD_DIM,
           "KV layer shape mismatch")

@@ -521,6 +521,11 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
             raise RuntimeError(f"{what} failed with status {rc}")
 
     plan = fused_plan(model, M)
+    # wider blocks keep the ten-launch layer; BONSAI_ROPE_IN_ATTENTION=1 drops its q / k norm + RoPE
+    # launch (same bits; measured slower at nine rows, where every workgroup of the attention
+    # repeats sixteen q rows)
+    rope_in_attention = (M <= decode_ops.ROPE_FUSED_MAX_WIDTH
+                         and os.environ.get("BONSAI_ROPE_IN_ATTENTION", "0") == "1")
     h_cur, h_nxt = ws.h[0][:M], ws.h[1][:M]
     torch.index_select(model.embed, 0, io.tokens, out=h_cur)
     for i, lw in enumerate(model.layers):
@@ -562,11 +567,17 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
                   "bonsai_add_rmsnorm_quant_int8")
             h_cur, h_nxt = h_nxt, h_cur
         _gemv(ws.a_q, ws.a_s, lw.wqkv, ws.xqkv, M, stream)
-        decode_ops.qk_norm_rope_kv_write(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
-                                         io.positions, ws.q[:M], kv[0, i], kv[1, i],
-                                         args.n_heads, args.n_kv_heads, sigma)
-        decode_ops.decode_attention(ws.q[:M], kv[0, i], kv[1, i], io.meta, ws.attn_scratch, sigma,
-                                    out_q=ws.o_q[:M], out_s=ws.o_s[:M])
+        if rope_in_attention:
+            decode_ops.decode_attention_rope(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
+                                             io.positions, kv[0, i], kv[1, i], io.meta,
+                                             ws.attn_scratch, sigma, args.n_heads,
+                                             out_q=ws.o_q[:M], out_s=ws.o_s[:M])
+        else:
+            decode_ops.qk_norm_rope_kv_write(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
+                                             io.positions, ws.q[:M], kv[0, i], kv[1, i],
+                                             args.n_heads, args.n_kv_heads, sigma)
+            decode_ops.decode_attention(ws.q[:M], kv[0, i], kv[1, i], io.meta, ws.attn_scratch, sigma,
+                                        out_q=ws.o_q[:M], out_s=ws.o_s[:M])
         _gemv(ws.o_q, ws.o_s, lw.wo, ws.attn_out, M, stream)
         check(actq.bonsai_add_rmsnorm_quant_int8(_vp(h_cur), _vp(ws.attn_out),
                                                  _vp(lw.post_attention_layernorm), eps, _vp(h_nxt),

@@ -94,14 +94,15 @@ int bonsai_decode_attention(const void *q, const void *k_layer, const void *v_la
                             int sigma, void *stream);
 
 /* bonsai_qk_norm_rope_kv_write and bonsai_decode_attention as one call (two launches instead of
- * three) for blocks of one or two rows: the chunk pass of the attention derives its q rows and
+ * three): the chunk pass of the attention derives its q rows and
  * the block's own K / V rows from the merged projection itself, with the arithmetic and rounding
  * points stated for bonsai_qk_norm_rope_kv_write (same bits), uses them without a round trip
  * through the cache, and writes the K / V rows to slots sigma .. sigma + M - 1 for later steps.
  * No counterpart in the reference beyond the two functions this stands for (model.py:388-436
  * and :996-1004); a one-token decode step spends as long on the separate RoPE launch as on the
- * attention itself.  Operands as for those two functions; always the matrix-core chunk pass;
- * M <= 2 (BONSAI_DECODE_ERR_ARG otherwise: use the two calls). */
+ * attention itself, while for blocks of nine rows the two calls are the faster form (every
+ * workgroup of the chunk pass repeats the q rows of its tile).  Operands as for those two
+ * functions; always the matrix-core chunk pass. */
 int bonsai_decode_attention_rope(const void *xqkv, const void *q_norm_w, const void *k_norm_w,
                                  float eps, const void *cos_table, const void *sin_table,
                                  const int32_t *positions, int max_pos, void *k_layer, void *v_layer,

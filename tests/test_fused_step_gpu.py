@@ -324,29 +324,42 @@ def test_argument_checks():
 
 
 ROPE_CASES = [
-    # M, n_heads, n_kv, sigma, cache_len, role
-    (1, 16, 8, 1024, 500, "ar"),
-    (1, 16, 8, 1024, 0, "ar"),        # nothing but the row itself
-    (1, 16, 8, 1024, 63, "ar"),       # the row is the last slot of a chunk
-    (1, 16, 8, 1024, 64, "ar"),       # ... the first slot of the next
-    (2, 16, 8, 1024, 63, "ar"),       # the two rows sit in two chunks (and two workgroups)
-    (2, 32, 8, 4096, 1531, "ar"),     # four query heads per kv head
-    (1, 32, 8, 4096, 4095, "ar"),
-    (2, 4, 2, 256, 255, "verify"),
-    (1, 6, 2, 64, 17, "ar"),
+    # M, n_heads, n_kv, sigma, cache_len, role, pending rows (draft roles)
+    (1, 16, 8, 1024, 500, "ar", 0),
+    (1, 16, 8, 1024, 0, "ar", 0),        # nothing but the row itself
+    (1, 16, 8, 1024, 63, "ar", 0),       # the row is the last slot of a chunk
+    (1, 16, 8, 1024, 64, "ar", 0),       # ... the first slot of the next
+    (2, 16, 8, 1024, 63, "ar", 0),       # the two rows sit in two chunks (and two workgroups)
+    (2, 32, 8, 4096, 1531, "ar", 0),     # four query heads per kv head
+    (1, 32, 8, 4096, 4095, "ar", 0),
+    (2, 4, 2, 256, 255, "verify", 0),
+    (1, 6, 2, 64, 17, "ar", 0),
+    # wide blocks: several pair tiles per kv head, more rows than a wave takes at a time
+    (9, 16, 8, 1024, 500, "verify", 0),
+    (9, 16, 8, 1024, 500, "draft", 1),
+    (9, 32, 8, 4096, 2000, "draft", 0),
+    (9, 16, 8, 1024, 60, "verify", 0),   # the block's rows straddle two chunks
+    (8, 16, 8, 1024, 0, "draft", 0),     # no history at all
+    (17, 16, 8, 1024, 1007, "draft", 9),
+    (17, 32, 8, 4096, 4079, "ar", 0),
+    (16, 6, 2, 64, 48, "draft", 3),
+    (5, 4, 2, 256, 100, "ar", 0),
+    (3, 16, 8, 1024, 126, "ar", 0),
+    (32, 16, 8, 1024, 300, "ar", 0),     # the widest block the library takes
 ]
 
 
-@pytest.mark.parametrize("M,n_heads,n_kv,sigma,cache_len,role", ROPE_CASES)
-def test_attention_with_rope_inside_gives_the_bits_of_the_two_calls(M, n_heads, n_kv, sigma, cache_len, role):
+@pytest.mark.parametrize("M,n_heads,n_kv,sigma,cache_len,role,n_pend", ROPE_CASES)
+def test_attention_with_rope_inside_gives_the_bits_of_the_two_calls(M, n_heads, n_kv, sigma, cache_len, role,
+                                                                    n_pend):
     """bonsai_decode_attention_rope against bonsai_qk_norm_rope_kv_write + bonsai_decode_attention:
     the bf16 and the quantised attention output and the K / V rows it leaves in the cache are the
     same bits; no other cache row is touched."""
     from bitmtp_amd import decode_ops, runtime
     print(f"[case] attention with rope inside M={M} heads={n_heads}/{n_kv} sigma={sigma} "
-          f"cache_len={cache_len} {role}", flush=True)
+          f"cache_len={cache_len} {role} pending={n_pend}", flush=True)
     gen = _gen(M + n_heads + sigma + cache_len)
-    slots = sigma + 17
+    slots = sigma + 32
     hd = 128
     xqkv = _rows(gen, M, (n_heads + 2 * n_kv) * hd, 1.5)
     qw = (1.0 + 0.1 * torch.randn(hd, generator=gen, device=DEV)).to(torch.bfloat16)
@@ -354,9 +367,11 @@ def test_attention_with_rope_inside_gives_the_bits_of_the_two_calls(M, n_heads, 
     max_pos = 8192
     ang = torch.rand(max_pos, hd, generator=gen, device=DEV) * 6.28
     cos, sin = torch.cos(ang).to(torch.bfloat16), torch.sin(ang).to(torch.bfloat16)
-    positions = torch.tensor([cache_len + i for i in range(M)], dtype=torch.int32, device=DEV)
+    # a verify block replays the anchor at cache_len - 1; the other roles start at cache_len
+    first = cache_len - 1 if role == "verify" else cache_len
+    positions = torch.tensor([first + i for i in range(M)], dtype=torch.int32, device=DEV)
     kv0 = (torch.randn(2, n_kv, slots, hd, generator=gen, device=DEV) * 1.2).to(torch.bfloat16)
-    meta = torch.tensor(runtime.step_descriptor(role, M, 8, cache_len, 0), dtype=torch.int32, device=DEV)
+    meta = torch.tensor(runtime.step_descriptor(role, M, 8, cache_len, n_pend), dtype=torch.int32, device=DEV)
     scratch = torch.empty(decode_ops.attention_scratch_bytes(M, n_heads, slots) // 4, dtype=torch.float32,
                           device=DEV)
 
@@ -385,17 +400,18 @@ def test_attention_with_rope_inside_gives_the_bits_of_the_two_calls(M, n_heads, 
     assert not changed[:, :, :sigma].any() and not changed[:, :, sigma + M:].any()
 
 
-def test_attention_with_rope_inside_refuses_wide_blocks():
+def test_attention_with_rope_inside_refuses_blocks_beyond_the_widest():
     from bitmtp_amd import decode_ops
-    xqkv = torch.zeros(3, (4 + 4) * 128, dtype=torch.bfloat16, device=DEV)
+    m = decode_ops.ROPE_FUSED_MAX_WIDTH + 1
+    xqkv = torch.zeros(m, (4 + 4) * 128, dtype=torch.bfloat16, device=DEV)
     w = torch.ones(128, dtype=torch.bfloat16, device=DEV)
     tab = torch.ones(16, 128, dtype=torch.bfloat16, device=DEV)
-    kv = torch.zeros(2, 2, 80, 128, dtype=torch.bfloat16, device=DEV)
+    kv = torch.zeros(2, 2, 128, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError):
-        decode_ops.decode_attention_rope(xqkv, w, w, EPS, tab, tab, torch.zeros(3, dtype=torch.int32, device=DEV),
-                                         kv[0], kv[1], torch.zeros(5, dtype=torch.int32, device=DEV),
-                                         torch.zeros(1 << 16, dtype=torch.float32, device=DEV), 64, 4,
-                                         out_bf16=torch.zeros(3, 512, dtype=torch.bfloat16, device=DEV))
+        decode_ops.decode_attention_rope(xqkv, w, w, EPS, tab, tab, torch.zeros(m, dtype=torch.int32, device=DEV),
+                                         kv[0], kv[1], torch.zeros(2 + m, dtype=torch.int32, device=DEV),
+                                         torch.zeros(1 << 18, dtype=torch.float32, device=DEV), 64, 4,
+                                         out_bf16=torch.zeros(m, 512, dtype=torch.bfloat16, device=DEV))
 
 
 @pytest.mark.parametrize("kind", ["t2g128", "q1"])
@@ -421,3 +437,28 @@ def test_decode_loop_tokens_do_not_depend_on_the_fused_layers(kind, monkeypatch)
         del atlas
     assert runs["1"][0] == runs["0"][0]
     assert _same_bits(runs["1"][1], runs["0"][1])
+
+
+@pytest.mark.parametrize("threshold,hybrid_m", [(0.9, None), (0.0, 1)])
+def test_hybrid_decode_tokens_do_not_depend_on_where_the_rope_runs(threshold, hybrid_m, monkeypatch):
+    """Hybrid decoding (draft and verify blocks of nine and more rows) through graphs whose
+    attention derives q / k itself and through graphs with the separate q / k launch commits the
+    same tokens, and the last step leaves the same logits bits."""
+    from bitmtp_amd import generate
+    from bitmtp_amd.model import BonsaiDecoder, ModelArgs
+    from bitmtp_amd.runtime import GraphAtlas
+    args = ModelArgs(dim=512, n_layers=3, n_heads=4, n_kv_heads=2, ffn_dim=1024, vocab_size=1000,
+                     mask_token_id=999)
+    model = BonsaiDecoder.random_init(args, seed=23, device=DEV)
+    prompt = np.random.default_rng(9).integers(0, 999, 19).tolist()
+    runs = {}
+    for flag in ("1", "0"):
+        monkeypatch.setenv("BONSAI_ROPE_IN_ATTENTION", flag)
+        atlas = GraphAtlas(model, segment_ladder=(128,), threshold=0.9)
+        print(f"[case] hybrid decode threshold={threshold} BONSAI_ROPE_IN_ATTENTION={flag}", flush=True)
+        toks, st = generate.hybrid_generate(atlas, prompt, threshold=threshold, hybrid_m=hybrid_m,
+                                            max_gen_len=40)
+        runs[flag] = (toks, st["n_iters"], atlas.workspace.logits.clone())
+        del atlas
+    assert runs["1"][0] == runs["0"][0] and runs["1"][1] == runs["0"][1]
+    assert _same_bits(runs["1"][2], runs["0"][2])
