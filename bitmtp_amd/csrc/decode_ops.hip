@@ -318,6 +318,87 @@ __device__ __forceinline__ attn_bf16x8_t attn_as_bf16x8(const uint4 v) {
     return r;
 }
 
+template <int CTRL>
+__device__ __forceinline__ float row_share(float v) {
+    const int x = __float_as_int(v);
+    return __int_as_float(__builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false));
+}
+
+// The merge of the partials of one (row, head): the 16 lanes of a DPP row hold the head, lane j
+// dims 8 j .. + 8 of every live partial and the statistics of part j.  num = sum over the parts,
+// in ascending order, of weight x accumulator, the weights normalised over the parts.
+//
+// DEVICE_SCOPE: the partials were stored by other workgroups of the SAME launch (device-scope
+// stores, part_store below): the loads carry the device scope too, so that no L2 of another XCD's
+// making is trusted for them.
+constexpr int kBufferWord3 = 0x00020000;   // raw buffer, 32-bit format, range check on
+constexpr int kDeviceScope = 16;           // cache-policy bit sc1 of buffer loads and stores
+
+// `hbase` = part + head_off floats; with DEVICE_SCOPE `part` and `part_bytes` must be uniform.
+template <bool DEVICE_SCOPE>
+__device__ __forceinline__ void combine_head_slice(const float *part, int part_bytes, int head_off, int live,
+                                                   int j, float (&num)[8]) {
+    const float *hbase = part + head_off;
+    // this thread's 8 dims of every live partial, and part j's statistics
+    float4 x0[kMaxParts], x1[kMaxParts];
+    float2 ml = make_float2(-INFINITY, 0.0f);
+    if constexpr (DEVICE_SCOPE) {
+        typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+        typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(part), 0, part_bytes, kBufferWord3);
+#pragma unroll
+        for (int c = 0; c < kMaxParts; ++c) {
+            if (c < live) {  // uniform
+                const int off = (head_off + c * kPartStride + 8 * j) * 4;
+                const v4u a = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kDeviceScope);
+                const v4u b = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off + 16, 0, kDeviceScope);
+                x0[c] = make_float4(__uint_as_float(a.x), __uint_as_float(a.y), __uint_as_float(a.z),
+                                    __uint_as_float(a.w));
+                x1[c] = make_float4(__uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z),
+                                    __uint_as_float(b.w));
+            }
+        }
+        if (j < live) {
+            const v2u t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (head_off + j * kPartStride + kHd) * 4, 0, kDeviceScope);
+            ml = make_float2(__uint_as_float(t.x), __uint_as_float(t.y));
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < kMaxParts; ++c) {
+            if (c < live) {  // uniform
+                const float4 *src = reinterpret_cast<const float4 *>(hbase + (size_t)c * kPartStride + 8 * j);
+                x0[c] = src[0];
+                x1[c] = src[1];
+            }
+        }
+        if (j < live) ml = *reinterpret_cast<const float2 *>(hbase + (size_t)j * kPartStride + kHd);
+    }
+
+    const float mx = bonsai_wave::max16(ml.x);
+    const float e = (ml.x == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ml.x - mx);
+    const float den = bonsai_wave::sum16(e * ml.y);
+    const float wj = e * (den > 0.0f ? 1.0f / den : 0.0f);  // weight of part j
+
+#pragma unroll
+    for (int i = 0; i < 8; ++i) num[i] = 0.0f;
+#define BONSAI_COMBINE_PART(C)                                                      \
+    {                                                                               \
+        const float wc = row_share<0x150 + (C)>(wj);                                \
+        if ((C) < live) {                                                           \
+            num[0] = fmaf(wc, x0[C].x, num[0]); num[1] = fmaf(wc, x0[C].y, num[1]); \
+            num[2] = fmaf(wc, x0[C].z, num[2]); num[3] = fmaf(wc, x0[C].w, num[3]); \
+            num[4] = fmaf(wc, x1[C].x, num[4]); num[5] = fmaf(wc, x1[C].y, num[5]); \
+            num[6] = fmaf(wc, x1[C].z, num[6]); num[7] = fmaf(wc, x1[C].w, num[7]); \
+        }                                                                           \
+    }
+    BONSAI_COMBINE_PART(0) BONSAI_COMBINE_PART(1) BONSAI_COMBINE_PART(2) BONSAI_COMBINE_PART(3)
+    BONSAI_COMBINE_PART(4) BONSAI_COMBINE_PART(5) BONSAI_COMBINE_PART(6) BONSAI_COMBINE_PART(7)
+    BONSAI_COMBINE_PART(8) BONSAI_COMBINE_PART(9) BONSAI_COMBINE_PART(10) BONSAI_COMBINE_PART(11)
+    BONSAI_COMBINE_PART(12) BONSAI_COMBINE_PART(13) BONSAI_COMBINE_PART(14) BONSAI_COMBINE_PART(15)
+#undef BONSAI_COMBINE_PART
+}
+
 // live parts of a step: the live chunks split into runs of ceil(live / parts)
 __host__ __device__ inline int attn_chunks_per_part(int live_chunks, int parts) {
     return (live_chunks + parts - 1) / parts;
@@ -325,8 +406,8 @@ __host__ __device__ inline int attn_chunks_per_part(int live_chunks, int parts) 
 
 // ROPE: the launch takes the merged q|k|v projection instead of finished q rows and does the work
 // of qk_norm_rope_kernel itself (a decode step of one token spends as long on that launch as on
-// this one).  Every workgroup derives the q rows of its pair tile -- one wave per (token, head) row, the very arithmetic of qk_norm_rope_kernel --
-// and hands them to its waves through LDS; a workgroup whose chunks reach the block's own rows
+// this one).  Every workgroup derives the q rows of its pair tile -- one wave per (token, head)
+// row, the very arithmetic of qk_norm_rope_kernel -- and hands them to its waves through LDS; a workgroup whose chunks reach the block's own rows
 // (logical index >= cache_len) derives those K rows the same way and takes the V rows from the
 // projection, never from the cache, so no workgroup uses what another one writes; the workgroup
 // of pair tile 0 that owns a row's chunk also writes it to the cache for the steps to come.
@@ -337,11 +418,26 @@ struct RopeIn {
     int max_pos;
 };
 
-template <bool ROPE>
+// FIN: no second launch.  A workgroup makes its partials visible to the device and counts itself
+// in on its kv head's arrival counter; the one that finds all the others there merges the
+// partials of its pair tile (combine_head_slice, what attn_combine_parts_kernel does), stores the
+// rows as bf16 with one maximum of |value| per (row, kv head) -- the parts a projection with the
+// maxima prologue quantises from -- and puts the counter back to zero.  Nobody waits.  Single
+// pair tile only (M x heads per kv head <= 16).
+struct FinOut {
+    unsigned *arrivals;   // [n_kv], zero between launches
+    uint16_t *out;        // bf16 [M, n_heads x 128]
+    uint16_t *amax;       // bf16 [M, amax_ld]: entries n_kv .. amax_ld - 1 are set to zero
+    int amax_ld;
+};
+
+template <bool ROPE, bool FIN>
 __global__ void __launch_bounds__(kAttnWaves * 64)
 attn_mfma_kernel(const uint16_t *q, uint16_t *k_layer, uint16_t *v_layer,
                  const int32_t *meta, float *part_out, float scale_log2e, int M, int n_heads,
-                 int n_kv, int G, int slots, int sigma, int parts, const RopeIn rope) {
+                 int n_kv, int G, int slots, int sigma, int parts, const RopeIn rope, const FinOut fin) {
+    __shared__ unsigned fin_last;
+    __shared__ float fin_max[kPairTile];
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kChunk * kVPitch];
     __shared__ __attribute__((aligned(16))) uint16_t q_new[ROPE ? kPairTile : 1][kHd];
     __shared__ __attribute__((aligned(16))) uint16_t k_new[ROPE ? BONSAI_MAX_WIDTH : 1][kHd];
@@ -645,18 +741,83 @@ attn_mfma_kernel(const uint16_t *q, uint16_t *k_layer, uint16_t *v_layer,
     }
 
     // acc_o[x][r]: pair 4 kb + r, dim 32 w + 16 x + col, unnormalised against m_run
+    const int part_bytes = M * n_heads * parts * kPartStride * 4;  // (the launcher keeps it below 2^31)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         if (valid[r]) {
-            float *dst = part_out +
-                         (((size_t)row_of[r] * n_heads + head_of[r]) * parts + part) * kPartStride;
-            dst[32 * w + col] = acc_o[0][r];
-            dst[32 * w + 16 + col] = acc_o[1][r];
-            if (w == 0 && col == 0) {
-                dst[kHd] = m_run[r];
-                dst[kHd + 1] = l_run[r];
+            const int rec = ((row_of[r] * n_heads + head_of[r]) * parts + part) * kPartStride;
+            float *dst = part_out + rec;
+            if constexpr (FIN) {  // device-scope stores: written through to where every XCD reads
+                const __amdgpu_buffer_rsrc_t rsrc =
+                    __builtin_amdgcn_make_buffer_rsrc(part_out, 0, part_bytes, kBufferWord3);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc_o[0][r]), rsrc,
+                                                      (rec + 32 * w + col) * 4, 0, kDeviceScope);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc_o[1][r]), rsrc,
+                                                      (rec + 32 * w + 16 + col) * 4, 0, kDeviceScope);
+                if (w == 0 && col == 0) {
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(m_run[r]), rsrc, (rec + kHd) * 4, 0,
+                                                          kDeviceScope);
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(l_run[r]), rsrc,
+                                                          (rec + kHd + 1) * 4, 0, kDeviceScope);
+                }
+            } else {
+                dst[32 * w + col] = acc_o[0][r];
+                dst[32 * w + 16 + col] = acc_o[1][r];
+                if (w == 0 && col == 0) {
+                    dst[kHd] = m_run[r];
+                    dst[kHd + 1] = l_run[r];
+                }
             }
         }
+    }
+    if constexpr (FIN) {
+        // The partials went out as device-scope stores, and a wave's store counter reaches zero
+        // when they have arrived: that wait stands for the release fence, whose write-back of
+        // the whole L2 costs each of the launch's waves its turn at it (tens of ns apiece, one
+        // after the other).  The arrival itself and the finisher's loads carry the device scope
+        // as well, so nothing else needs to be written back or invalidated.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const int live = (live_chunks + cpw - 1) / cpw;  // workgroups of this kv head that got here
+        if (threadIdx.x == 0) {
+            const unsigned old = __hip_atomic_fetch_add(&fin.arrivals[kvh], 1u, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+            fin_last = old == (unsigned)(live - 1) ? 1u : 0u;
+        }
+        __syncthreads();
+        if (!fin_last) return;
+        // thread = (pair of the tile, 8 dims); the pairs of a row are neighbours
+        const int pr = threadIdx.x >> 4, j = threadIdx.x & 15;
+        const bool mine = pr < pairs_total;
+        const int pc = mine ? pr : pairs_total - 1;
+        const int row = pc / G, head = kvh * G + (pc - row * G);
+        float num[8];
+        combine_head_slice<true>(part_out, part_bytes, (row * n_heads + head) * parts * kPartStride, live, j, num);
+        uint32_t ob[8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float o = bf16_round(num[i]);
+            ob[i] = f32_to_bf16_bits(o);
+            amax = fmaxf(amax, fabsf(o));
+        }
+        if (mine)
+            reinterpret_cast<uint4 *>(fin.out + ((size_t)row * n_heads + head) * kHd)[j] =
+                make_uint4(ob[0] | (ob[1] << 16), ob[2] | (ob[3] << 16), ob[4] | (ob[5] << 16),
+                           ob[6] | (ob[7] << 16));
+        amax = bonsai_wave::max16(amax);
+        if (j == 0) fin_max[pr] = mine ? amax : 0.0f;
+        __syncthreads();
+        if ((int)threadIdx.x < M) {  // one thread per row: the maximum over the row's heads of this kv head
+            float top = 0.0f;
+            for (int g = 0; g < G; ++g) top = fmaxf(top, fin_max[threadIdx.x * G + g]);
+            uint16_t *arow = fin.amax + (size_t)threadIdx.x * fin.amax_ld;
+            arow[kvh] = (uint16_t)f32_to_bf16_bits(top);  // exact: one of the bf16 values stored
+            if (kvh == n_kv - 1)
+                for (int x = n_kv; x < fin.amax_ld; ++x) arow[x] = 0;
+        }
+        if (threadIdx.x == 0)
+            __hip_atomic_store(&fin.arrivals[kvh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -793,12 +954,6 @@ attn_combine_kernel(const float *ppart, const int32_t *pmeta, uint16_t *pout, in
 // long.  Accumulation runs over the parts in ascending order.
 constexpr int kCombinePartsThreads = 512;
 
-template <int CTRL>
-__device__ __forceinline__ float row_share(float v) {
-    const int x = __float_as_int(v);
-    return __int_as_float(__builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false));
-}
-
 __global__ void __launch_bounds__(kCombinePartsThreads)
 attn_combine_parts_kernel(const float *part, const int32_t *meta, uint16_t *out_bf16, int8_t *out_q,
                           float *out_s, int M, int n_heads, int parts, int sigma) {
@@ -813,44 +968,8 @@ attn_combine_parts_kernel(const float *part, const int32_t *meta, uint16_t *out_
     const bool mine = tid < nvec;
     const int v = mine ? tid : nvec - 1;
     const int head = v >> 4, j = v & 15;
-    const float *hbase = part + ((size_t)m * n_heads + head) * parts * kPartStride;
-
-    // this thread's 8 dims of every live partial, and part j's statistics
-    float4 x0[kMaxParts], x1[kMaxParts];
-#pragma unroll
-    for (int c = 0; c < kMaxParts; ++c) {
-        if (c < live) {  // uniform
-            const float4 *src = reinterpret_cast<const float4 *>(hbase + (size_t)c * kPartStride + 8 * j);
-            x0[c] = src[0];
-            x1[c] = src[1];
-        }
-    }
-    float2 ml = make_float2(-INFINITY, 0.0f);
-    if (j < live) ml = *reinterpret_cast<const float2 *>(hbase + (size_t)j * kPartStride + kHd);
-
-    const float mx = bonsai_wave::max16(ml.x);
-    const float e = (ml.x == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ml.x - mx);
-    const float den = bonsai_wave::sum16(e * ml.y);
-    const float wj = e * (den > 0.0f ? 1.0f / den : 0.0f);  // weight of part j
-
     float num[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) num[i] = 0.0f;
-#define BONSAI_COMBINE_PART(C)                                                      \
-    {                                                                               \
-        const float wc = row_share<0x150 + (C)>(wj);                                \
-        if ((C) < live) {                                                           \
-            num[0] = fmaf(wc, x0[C].x, num[0]); num[1] = fmaf(wc, x0[C].y, num[1]); \
-            num[2] = fmaf(wc, x0[C].z, num[2]); num[3] = fmaf(wc, x0[C].w, num[3]); \
-            num[4] = fmaf(wc, x1[C].x, num[4]); num[5] = fmaf(wc, x1[C].y, num[5]); \
-            num[6] = fmaf(wc, x1[C].z, num[6]); num[7] = fmaf(wc, x1[C].w, num[7]); \
-        }                                                                           \
-    }
-    BONSAI_COMBINE_PART(0) BONSAI_COMBINE_PART(1) BONSAI_COMBINE_PART(2) BONSAI_COMBINE_PART(3)
-    BONSAI_COMBINE_PART(4) BONSAI_COMBINE_PART(5) BONSAI_COMBINE_PART(6) BONSAI_COMBINE_PART(7)
-    BONSAI_COMBINE_PART(8) BONSAI_COMBINE_PART(9) BONSAI_COMBINE_PART(10) BONSAI_COMBINE_PART(11)
-    BONSAI_COMBINE_PART(12) BONSAI_COMBINE_PART(13) BONSAI_COMBINE_PART(14) BONSAI_COMBINE_PART(15)
-#undef BONSAI_COMBINE_PART
+    combine_head_slice<false>(part, 0, (m * n_heads + head) * parts * kPartStride, live, j, num);
 
     float o[8];
     float amax = 0.0f;
@@ -1452,10 +1571,10 @@ extern "C" int64_t bonsai_decode_attention_scratch_bytes(int M, int n_heads, int
 static int launch_attention(const void *q, void *k_layer, void *v_layer, const int32_t *meta,
                             void *scratch, void *out_bf16, int8_t *out_q, float *out_s, float scale,
                             int M, int n_heads, int n_kv, int slots, int sigma, const RopeIn *rope,
-                            hipStream_t st) {
+                            const FinOut *fin, hipStream_t st) {
     if (!q || !k_layer || !v_layer || !meta || !scratch) return BONSAI_DECODE_ERR_ARG;
     if ((out_q == nullptr) != (out_s == nullptr)) return BONSAI_DECODE_ERR_ARG;
-    if (!out_bf16 && !out_q) return BONSAI_DECODE_ERR_ARG;
+    if (!fin && !out_bf16 && !out_q) return BONSAI_DECODE_ERR_ARG;
     if (M < 1 || M > BONSAI_MAX_WIDTH || n_kv < 1 || n_heads < n_kv || n_heads % n_kv != 0 ||
         n_heads > kCombineMaxHeads || sigma < 0 || sigma + M > slots ||
         (sigma + M + kChunk - 1) / kChunk > kCombineMaxChunks)
@@ -1480,16 +1599,23 @@ static int launch_attention(const void *q, void *k_layer, void *v_layer, const i
         parts = a.n_chunks < kMaxParts ? a.n_chunks : kMaxParts;
         const int tiles = (M * a.hpg + kPairTile - 1) / kPairTile;
         const dim3 grid(n_kv * parts * tiles), block(kAttnWaves * 64);
+        if (fin != nullptr) {  // the one launch that also merges its partials (rope != nullptr, one tile)
+            hipLaunchKernelGGL((attn_mfma_kernel<true, true>), grid, block, 0, st,
+                               static_cast<const uint16_t *>(q), static_cast<uint16_t *>(k_layer),
+                               static_cast<uint16_t *>(v_layer), meta, a.part, a.scale_log2e, M,
+                               n_heads, n_kv, a.hpg, slots, sigma, parts, *rope, *fin);
+            return hipGetLastError() == hipSuccess ? BONSAI_DECODE_OK : BONSAI_DECODE_ERR_LAUNCH;
+        }
         if (rope != nullptr)
-            hipLaunchKernelGGL(attn_mfma_kernel<true>, grid, block, 0, st,
+            hipLaunchKernelGGL((attn_mfma_kernel<true, false>), grid, block, 0, st,
                                static_cast<const uint16_t *>(q), static_cast<uint16_t *>(k_layer),
                                static_cast<uint16_t *>(v_layer), meta, a.part, a.scale_log2e, M,
-                               n_heads, n_kv, a.hpg, slots, sigma, parts, *rope);
+                               n_heads, n_kv, a.hpg, slots, sigma, parts, *rope, FinOut{});
         else
-            hipLaunchKernelGGL(attn_mfma_kernel<false>, grid, block, 0, st,
+            hipLaunchKernelGGL((attn_mfma_kernel<false, false>), grid, block, 0, st,
                                static_cast<const uint16_t *>(q), static_cast<uint16_t *>(k_layer),
                                static_cast<uint16_t *>(v_layer), meta, a.part, a.scale_log2e, M,
-                               n_heads, n_kv, a.hpg, slots, sigma, parts, RopeIn{});
+                               n_heads, n_kv, a.hpg, slots, sigma, parts, RopeIn{}, FinOut{});
     } else {
     const int rw = rows_per_wave(M);
     a.row_groups = (M + rw - 1) / rw;
@@ -1535,7 +1661,7 @@ extern "C" int bonsai_decode_attention(const void *q, const void *k_layer, const
                                        int8_t *out_q, float *out_s, float scale, int M, int n_heads,
                                        int n_kv, int slots, int sigma, void *stream) {
     return launch_attention(q, const_cast<void *>(k_layer), const_cast<void *>(v_layer), meta, scratch,
-                            out_bf16, out_q, out_s, scale, M, n_heads, n_kv, slots, sigma, nullptr,
+                            out_bf16, out_q, out_s, scale, M, n_heads, n_kv, slots, sigma, nullptr, nullptr,
                             static_cast<hipStream_t>(stream));
 }
 
@@ -1552,7 +1678,30 @@ extern "C" int bonsai_decode_attention_rope(const void *xqkv, const void *q_norm
                       static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table),
                       positions, eps, max_pos};
     return launch_attention(xqkv, k_layer, v_layer, meta, scratch, out_bf16, out_q, out_s, scale, M,
-                            n_heads, n_kv, slots, sigma, &rope, static_cast<hipStream_t>(stream));
+                            n_heads, n_kv, slots, sigma, &rope, nullptr, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int bonsai_decode_attention_rope_parts(const void *xqkv, const void *q_norm_w,
+                                                  const void *k_norm_w, float eps, const void *cos_table,
+                                                  const void *sin_table, const int32_t *positions,
+                                                  int max_pos, void *k_layer, void *v_layer,
+                                                  const int32_t *meta, void *scratch, void *arrivals,
+                                                  void *out_bf16, void *out_amax, float scale, int M,
+                                                  int n_heads, int n_kv, int slots, int sigma,
+                                                  void *stream) {
+    if (!q_norm_w || !k_norm_w || !cos_table || !sin_table || !positions || max_pos < 1 || !arrivals ||
+        !out_bf16 || !out_amax)
+        return BONSAI_DECODE_ERR_ARG;
+    if (M < 1 || n_kv < 1 || n_heads < n_kv || n_heads % n_kv != 0 || M * (n_heads / n_kv) > kPairTile ||
+        n_kv > BONSAI_ATTN_MAX_KV_HEADS)
+        return BONSAI_DECODE_ERR_ARG;
+    const RopeIn rope{static_cast<const uint16_t *>(q_norm_w), static_cast<const uint16_t *>(k_norm_w),
+                      static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table),
+                      positions, eps, max_pos};
+    const FinOut fin{static_cast<unsigned *>(arrivals), static_cast<uint16_t *>(out_bf16),
+                     static_cast<uint16_t *>(out_amax), (n_kv + 7) & ~7};
+    return launch_attention(xqkv, k_layer, v_layer, meta, scratch, nullptr, nullptr, nullptr, scale, M,
+                            n_heads, n_kv, slots, sigma, &rope, &fin, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int bonsai_kv_commit(void *kv, int n_layers, int n_kv, int slots, int src_slot,

@@ -45,6 +45,9 @@ def load_decode_kernel() -> None:
     lib.bonsai_decode_attention_rope.argtypes = [vp, vp, vp, cf, vp, vp, vp, ci, vp, vp, vp, vp, vp, vp, vp,
                                                  cf, ci, ci, ci, ci, ci, vp]
     lib.bonsai_decode_attention_rope.restype = ci
+    lib.bonsai_decode_attention_rope_parts.argtypes = [vp, vp, vp, cf, vp, vp, vp, ci, vp, vp, vp, vp, vp,
+                                                       vp, vp, cf, ci, ci, ci, ci, ci, vp]
+    lib.bonsai_decode_attention_rope_parts.restype = ci
     lib.bonsai_decode_set_tuning.argtypes = [ci]
     lib.bonsai_decode_set_tuning.restype = None
     lib.bonsai_decode_set_attention_engine.argtypes = [ci]
@@ -217,6 +220,61 @@ def decode_attention_rope(xqkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: 
             _ptr(out_q), _ptr(out_s), float(scale), m, n_heads, n_kv, slots, int(sigma),
             _stream(xqkv.device))
     _need(rc == 0, f"bonsai_decode_attention_rope failed with status {rc}")
+
+
+ATTN_MAX_KV_HEADS = 64
+
+
+def attention_amax_ld(n_kv: int) -> int:
+    """Row pitch of the maxima :func:`decode_attention_rope_parts` leaves (one per kv head)."""
+    return (n_kv + 7) & ~7
+
+
+def decode_attention_rope_parts(xqkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: torch.Tensor,
+                                eps: float, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                                k_layer: torch.Tensor, v_layer: torch.Tensor, meta: torch.Tensor,
+                                scratch: torch.Tensor, arrivals: torch.Tensor, sigma: int, n_heads: int,
+                                out_bf16: torch.Tensor, out_amax: torch.Tensor,
+                                scale: Optional[float] = None) -> None:
+    """:func:`decode_attention_rope` in one launch: the last workgroup of every kv head merges the
+    partials itself and leaves the rows as bf16 plus one maximum per (row, kv head) in
+    ``out_amax [M, attention_amax_ld(n_kv)]`` -- what ``packed_gemv_fused(..., amax=out_amax,
+    parts=n_kv)`` quantises from, to the bits of the two-launch form.  ``arrivals``: int32
+    counters, one per kv head, zero before the first call (every call leaves them zero)."""
+    m = xqkv.shape[0]
+    n_kv, slots = k_layer.shape[0], k_layer.shape[1]
+    for t, name in ((xqkv, "xqkv"), (q_norm_w, "q_norm_w"), (k_norm_w, "k_norm_w"), (cos, "cos"),
+                    (sin, "sin"), (k_layer, "k_layer"), (v_layer, "v_layer"), (out_bf16, "out_bf16"),
+                    (out_amax, "out_amax")):
+        _check(t, torch.bfloat16, name)
+    _check(positions, torch.int32, "positions")
+    _check(meta, torch.int32, "meta")
+    _check(arrivals, torch.int32, "arrivals")
+    _need(n_heads % n_kv == 0 and 1 <= m and m * (n_heads // n_kv) <= 16,
+          "one pair tile only: rows x heads per kv head <= 16")
+    _need(n_kv <= ATTN_MAX_KV_HEADS and arrivals.numel() >= n_kv, "one arrival counter per kv head")
+    _need(xqkv.shape == (m, (n_heads + 2 * n_kv) * HEAD_DIM), "xqkv shape mismatch")
+    _need(k_layer.shape == v_layer.shape and k_layer.dim() == 3 and k_layer.shape[2] == HEAD_DIM,
+          "KV layer shape mismatch")
+    _need(cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == HEAD_DIM,
+          "RoPE table shape mismatch")
+    _need(positions.numel() == m and q_norm_w.numel() == HEAD_DIM and k_norm_w.numel() == HEAD_DIM,
+          "positions / norm weight size mismatch")
+    _need(meta.numel() >= 2 + m, "meta needs 2 + M entries")
+    _need(scratch.is_cuda and scratch.is_contiguous()
+          and scratch.numel() * scratch.element_size() >= attention_scratch_bytes(m, n_heads, slots),
+          "attention scratch too small")
+    _need(out_bf16.numel() == m * n_heads * HEAD_DIM, "out_bf16 size mismatch")
+    _need(out_amax.numel() >= m * attention_amax_ld(n_kv), "out_amax too small")
+    if scale is None:
+        scale = 1.0 / math.sqrt(HEAD_DIM)
+    with torch.cuda.device(xqkv.device):
+        rc = decode_lib().bonsai_decode_attention_rope_parts(
+            _ptr(xqkv), _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(cos), _ptr(sin), _ptr(positions),
+            cos.shape[0], _ptr(k_layer), _ptr(v_layer), _ptr(meta), _ptr(scratch), _ptr(arrivals),
+            _ptr(out_bf16), _ptr(out_amax), float(scale), m, n_heads, n_kv, slots, int(sigma),
+            _stream(xqkv.device))
+    _need(rc == 0, f"bonsai_decode_attention_rope_parts failed with status {rc}")
 
 
 def kv_commit(kv: torch.Tensor, src_slot: int, dst_slot: int, n: int) -> None:

@@ -370,6 +370,11 @@ class Workspace:
         self.inner = buf((m_max, args.ffn_dim), bf)
         self.inner_amax = buf((min(m_max, 2), 1024), bf)
         self.sumsq = buf((min(m_max, 2), 256), torch.float64)
+        # the attention that merges its own partials: rows as bf16, one maximum per kv head, and the
+        # arrival counters of its workgroups (zero between launches)
+        self.attn_rows = buf((min(m_max, 2), args.q_dim), bf)
+        self.attn_amax = buf((min(m_max, 2), decode_ops.attention_amax_ld(args.n_kv_heads)), bf)
+        self.attn_arrivals = buf((decode_ops.ATTN_MAX_KV_HEADS,), torch.int32)
         self.i_q = buf((m_max, args.ffn_dim), i8)
         self.i_s = buf((m_max,), f32)
         self.ffn_out = buf((m_max, args.dim), bf)
@@ -457,6 +462,7 @@ class FusedPlan:
     o: int      # o projection: sums of squares
     gu: int     # gate|up projection: maxima
     down: int   # down projection: sums of squares
+    attn: int = 0   # attention: maxima, one per kv head, when it merges its own partials (else 0)
 
 
 def fused_plan(model: "BonsaiDecoder", m: int) -> Optional[FusedPlan]:
@@ -477,6 +483,10 @@ def fused_plan(model: "BonsaiDecoder", m: int) -> Optional[FusedPlan]:
         down=ops.fused_parts(ops.EPI_ADD_SUMSQ, m, lw.w_down.out_features, lw.w_down.in_features, bits=bits))
     if min(plan.o, plan.gu, plan.down) < 1 or max(plan.o, plan.down) > 256 or plan.gu > 1024:
         return None
+    a = model.args
+    if (m * (a.n_heads // a.n_kv_heads) <= 16 and a.n_kv_heads <= decode_ops.ATTN_MAX_KV_HEADS
+            and os.environ.get("BONSAI_ATTENTION_ONE_LAUNCH", "1") != "0"):
+        plan.attn = a.n_kv_heads
     return plan
 
 
@@ -542,12 +552,22 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
                 _fused(lw.wqkv, M, stream, act=h_cur, act_aux=ws.sumsq, act_kind=ops.ACT_BF16_NORM,
                        act_parts=plan.down, norm_w=lw.input_layernorm, eps=eps, out=ws.xqkv,
                        epi=ops.EPI_PLAIN)
-            decode_ops.decode_attention_rope(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
-                                             io.positions, kv[0, i], kv[1, i], io.meta,
-                                             ws.attn_scratch, sigma, args.n_heads,
-                                             out_q=ws.o_q[:M], out_s=ws.o_s[:M])
-            _fused(lw.wo, M, stream, act=ws.o_q, act_aux=ws.o_s, act_kind=ops.ACT_INT8, out=h_nxt,
-                   epi=ops.EPI_ADD_SUMSQ, residual=h_cur, out_aux=ws.sumsq)
+            if plan.attn:
+                decode_ops.decode_attention_rope_parts(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
+                                                       io.positions, kv[0, i], kv[1, i], io.meta,
+                                                       ws.attn_scratch, ws.attn_arrivals, sigma,
+                                                       args.n_heads, ws.attn_rows[:M], ws.attn_amax)
+                _fused(lw.wo, M, stream, act=ws.attn_rows, act_aux=ws.attn_amax,
+                       act_kind=ops.ACT_BF16_AMAX, act_parts=plan.attn, out=h_nxt,
+                       epi=ops.EPI_ADD_SUMSQ, residual=h_cur, out_aux=ws.sumsq)
+            else:
+                decode_ops.decode_attention_rope(ws.xqkv[:M], lw.q_norm, lw.k_norm, eps, cos, sin,
+                                                 io.positions, kv[0, i], kv[1, i], io.meta,
+                                                 ws.attn_scratch, sigma, args.n_heads,
+                                                 out_q=ws.o_q[:M], out_s=ws.o_s[:M])
+                _fused(lw.wo, M, stream, act=ws.o_q, act_aux=ws.o_s,
+                       act_kind=ops.ACT_INT8, out=h_nxt, epi=ops.EPI_ADD_SUMSQ, residual=h_cur,
+                       out_aux=ws.sumsq)
             h_cur, h_nxt = h_nxt, h_cur
             _fused(lw.w_gu, M, stream, act=h_cur, act_aux=ws.sumsq, act_kind=ops.ACT_BF16_NORM,
                    act_parts=plan.o, norm_w=lw.post_attention_layernorm, eps=eps, out=ws.inner,

@@ -110,6 +110,28 @@ int bonsai_decode_attention_rope(const void *xqkv, const void *q_norm_w, const v
                                  float *out_s, float scale, int M, int n_heads, int n_kv, int slots,
                                  int sigma, void *stream);
 
+/* bonsai_decode_attention_rope in ONE launch, for a projection that quantises from bf16 rows
+ * and per-part maxima (t2g128_gemv_fused / q1g128_gemv_fused with BONSAI_ACT_BF16_AMAX, act_parts
+ * = n_kv; include/bonsai_gemv.h): the workgroup of a kv head that finishes last merges that kv
+ * head's partials itself (the arithmetic of the second launch) and stores
+ *   out_bf16 [M, n_heads x 128]            the attention rows, the bits of
+ *                                          bonsai_decode_attention(_rope)'s out_bf16;
+ *   out_amax bf16 [M, (n_kv + 7) & ~7]     entry [m, h]: max |out_bf16| over the heads of kv head h
+ *                                          (the rest zero), so that the projection's multiplier
+ *                                          is the out_s of the two-launch form, bit for bit.
+ * arrivals: n_kv 32-bit counters (BONSAI_ATTN_MAX_KV_HEADS at most) that are ZERO before the first
+ * call; every call leaves them zero.  Calls that share `arrivals` or `scratch` must not overlap.
+ * One pair tile only: M x (n_heads / n_kv) <= 16 (BONSAI_DECODE_ERR_ARG otherwise).  No
+ * counterpart in the reference, as for bonsai_decode_attention_rope. */
+#define BONSAI_ATTN_MAX_KV_HEADS 64
+int bonsai_decode_attention_rope_parts(const void *xqkv, const void *q_norm_w, const void *k_norm_w,
+                                       float eps, const void *cos_table, const void *sin_table,
+                                       const int32_t *positions, int max_pos, void *k_layer,
+                                       void *v_layer, const int32_t *meta, void *scratch,
+                                       void *arrivals, void *out_bf16, void *out_amax, float scale,
+                                       int M, int n_heads, int n_kv, int slots, int sigma,
+                                       void *stream);
+
 /* Copies n KV rows of every layer and kv head from slot src to slot dst inside one
  * shared buffer [2, n_layers, n_kv, slots, 128] bf16 (commit_kv / commit_kv_from_verify,
  * src/bonsai_sft/gpu/fast_runtime.py:467-508).  Source and destination ranges must

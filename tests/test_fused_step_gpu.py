@@ -462,3 +462,154 @@ def test_hybrid_decode_tokens_do_not_depend_on_where_the_rope_runs(threshold, hy
         del atlas
     assert runs["1"][0] == runs["0"][0] and runs["1"][1] == runs["0"][1]
     assert _same_bits(runs["1"][2], runs["0"][2])
+
+
+MERGE_CASES = [
+    # M, n_heads, n_kv, sigma, cache_len, role
+    (1, 16, 8, 1024, 500, "ar"),
+    (1, 16, 8, 1024, 0, "ar"),         # one live part
+    (1, 16, 8, 1024, 63, "ar"),
+    (1, 16, 8, 1024, 64, "ar"),
+    (2, 16, 8, 1024, 1022, "ar"),      # every part live
+    (2, 32, 8, 4096, 1531, "ar"),
+    (1, 32, 8, 4096, 4095, "ar"),      # runs of several chunks per part
+    (2, 4, 2, 256, 255, "verify"),
+    (1, 6, 2, 64, 17, "ar"),           # three heads per kv head
+    (2, 16, 16, 128, 100, "ar"),       # one head per kv head, sixteen counters
+    (8, 16, 8, 1024, 300, "draft"),    # a full pair tile
+    (4, 32, 8, 4096, 77, "ar"),
+]
+
+
+@pytest.mark.parametrize("M,n_heads,n_kv,sigma,cache_len,role", MERGE_CASES)
+def test_attention_that_merges_its_own_partials(M, n_heads, n_kv, sigma, cache_len, role):
+    """bonsai_decode_attention_rope_parts (one launch) against bonsai_decode_attention_rope (two):
+    the same bf16 rows, maxima whose largest gives the same multiplier, counters back at zero --
+    twice in a row on the same counters, the second time with a shorter history."""
+    from bitmtp_amd import decode_ops, runtime
+    print(f"[case] self-merging attention M={M} heads={n_heads}/{n_kv} sigma={sigma} "
+          f"cache_len={cache_len} {role}", flush=True)
+    gen = _gen(3 * M + n_heads + sigma + cache_len)
+    slots, hd = sigma + 32, 128
+    qw = (1.0 + 0.1 * torch.randn(hd, generator=gen, device=DEV)).to(torch.bfloat16)
+    kw = (1.0 + 0.1 * torch.randn(hd, generator=gen, device=DEV)).to(torch.bfloat16)
+    max_pos = 8192
+    ang = torch.rand(max_pos, hd, generator=gen, device=DEV) * 6.28
+    cos, sin = torch.cos(ang).to(torch.bfloat16), torch.sin(ang).to(torch.bfloat16)
+    scratch = torch.empty(decode_ops.attention_scratch_bytes(M, n_heads, slots) // 4, dtype=torch.float32,
+                          device=DEV)
+    arrivals = torch.zeros(decode_ops.ATTN_MAX_KV_HEADS, dtype=torch.int32, device=DEV)
+    ld = decode_ops.attention_amax_ld(n_kv)
+    for clen in (cache_len, cache_len // 3 + (1 if role == "verify" else 0)):
+        xqkv = _rows(gen, M, (n_heads + 2 * n_kv) * hd, 1.5)
+        first = clen - 1 if role == "verify" else clen
+        positions = torch.tensor([first + i for i in range(M)], dtype=torch.int32, device=DEV)
+        kv0 = (torch.randn(2, n_kv, slots, hd, generator=gen, device=DEV) * 1.2).to(torch.bfloat16)
+        meta = torch.tensor(runtime.step_descriptor(role, M, 8, clen, 0), dtype=torch.int32, device=DEV)
+        kv_a = kv0.clone()
+        o_a = torch.zeros(M, n_heads * hd, dtype=torch.bfloat16, device=DEV)
+        q_a = torch.zeros(M, n_heads * hd, dtype=torch.int8, device=DEV)
+        s_a = torch.zeros(M, dtype=torch.float32, device=DEV)
+        decode_ops.decode_attention_rope(xqkv, qw, kw, EPS, cos, sin, positions, kv_a[0], kv_a[1], meta,
+                                         scratch, sigma, n_heads, out_bf16=o_a, out_q=q_a, out_s=s_a)
+        torch.cuda.synchronize()
+        kv_b = kv0.clone()
+        o_b = torch.zeros_like(o_a)
+        amax = torch.full((M, ld), 7.0, dtype=torch.bfloat16, device=DEV)
+        scratch.fill_(float("nan"))
+        decode_ops.decode_attention_rope_parts(xqkv, qw, kw, EPS, cos, sin, positions, kv_b[0], kv_b[1],
+                                               meta, scratch, arrivals, sigma, n_heads, o_b, amax)
+        torch.cuda.synchronize()
+        assert _same_bits(o_a, o_b)
+        assert torch.equal(kv_a.view(torch.int16), kv_b.view(torch.int16))
+        assert int(arrivals.abs().sum()) == 0
+        assert float(amax[:, n_kv:].float().abs().sum()) == 0.0
+        per_kv = o_b.float().abs().view(M, n_kv, -1).amax(dim=2)
+        assert torch.equal(amax[:, :n_kv].float(), per_kv)
+        top = amax.float().amax(dim=1).clamp_min(1e-5)
+        assert torch.equal((1.0 / top) * 127.0, s_a)
+
+
+@pytest.mark.parametrize("bits", [2, 1])
+@pytest.mark.parametrize("M", [1, 2])
+def test_o_projection_from_the_self_merging_attention(M, bits):
+    """attention (one launch) -> o projection that quantises from its rows and maxima, against
+    attention (two launches, int8 rows out) -> o projection: the residual stream and the sums of
+    squares that come out are the same bits."""
+    from bitmtp_amd import decode_ops, ops, runtime
+    n_heads, n_kv, sigma, cache_len, hd = 16, 8, 1024, 700, 128
+    print(f"[case] o projection behind the self-merging attention M={M} bits={bits}", flush=True)
+    gen = _gen(50 + M + bits)
+    slots = sigma + 32
+    w_o = _packed(gen, n_heads * hd, n_heads * hd, bits)
+    xqkv = _rows(gen, M, (n_heads + 2 * n_kv) * hd, 1.5)
+    h = _rows(gen, M, n_heads * hd, 1.0)
+    qw = (1.0 + 0.1 * torch.randn(hd, generator=gen, device=DEV)).to(torch.bfloat16)
+    kw = (1.0 + 0.1 * torch.randn(hd, generator=gen, device=DEV)).to(torch.bfloat16)
+    ang = torch.rand(4096, hd, generator=gen, device=DEV) * 6.28
+    cos, sin = torch.cos(ang).to(torch.bfloat16), torch.sin(ang).to(torch.bfloat16)
+    positions = torch.tensor([cache_len + i for i in range(M)], dtype=torch.int32, device=DEV)
+    kv0 = (torch.randn(2, n_kv, slots, hd, generator=gen, device=DEV) * 1.2).to(torch.bfloat16)
+    meta = torch.tensor(runtime.step_descriptor("ar", M, 8, cache_len, 0), dtype=torch.int32, device=DEV)
+    scratch = torch.empty(decode_ops.attention_scratch_bytes(M, n_heads, slots) // 4, dtype=torch.float32,
+                          device=DEV)
+    kv_a = kv0.clone()
+    q_a = torch.zeros(M, n_heads * hd, dtype=torch.int8, device=DEV)
+    s_a = torch.zeros(M, dtype=torch.float32, device=DEV)
+    decode_ops.decode_attention_rope(xqkv, qw, kw, EPS, cos, sin, positions, kv_a[0], kv_a[1], meta, scratch,
+                                     sigma, n_heads, out_q=q_a, out_s=s_a)
+    h_a, ss_a, parts_a = ops.packed_gemv_fused(q_a, w_o.weight, w_o.weight_scale, bits=bits, s=s_a,
+                                               epi=ops.EPI_ADD_SUMSQ, residual=h)
+    kv_b = kv0.clone()
+    rows = torch.zeros(M, n_heads * hd, dtype=torch.bfloat16, device=DEV)
+    amax = torch.zeros(M, decode_ops.attention_amax_ld(n_kv), dtype=torch.bfloat16, device=DEV)
+    arrivals = torch.zeros(decode_ops.ATTN_MAX_KV_HEADS, dtype=torch.int32, device=DEV)
+    decode_ops.decode_attention_rope_parts(xqkv, qw, kw, EPS, cos, sin, positions, kv_b[0], kv_b[1], meta,
+                                           scratch, arrivals, sigma, n_heads, rows, amax)
+    s_b = torch.zeros(M, dtype=torch.float32, device=DEV)
+    h_b, ss_b, parts_b = ops.packed_gemv_fused(rows, w_o.weight, w_o.weight_scale, bits=bits, amax=amax,
+                                               parts=n_kv, epi=ops.EPI_ADD_SUMSQ, residual=h, s_out=s_b)
+    torch.cuda.synchronize()
+    assert parts_a == parts_b and torch.equal(s_a, s_b)
+    assert _same_bits(h_a, h_b)
+    assert torch.equal(ss_a[:M * parts_a].view(torch.int64), ss_b[:M * parts_b].view(torch.int64))
+
+
+def test_self_merging_attention_refuses_more_than_one_pair_tile():
+    from bitmtp_amd import decode_ops
+    m, n_heads, n_kv = 9, 4, 2     # 18 pairs
+    xqkv = torch.zeros(m, (n_heads + 2 * n_kv) * 128, dtype=torch.bfloat16, device=DEV)
+    w = torch.ones(128, dtype=torch.bfloat16, device=DEV)
+    tab = torch.ones(16, 128, dtype=torch.bfloat16, device=DEV)
+    kv = torch.zeros(2, n_kv, 128, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        decode_ops.decode_attention_rope_parts(
+            xqkv, w, w, EPS, tab, tab, torch.zeros(m, dtype=torch.int32, device=DEV), kv[0], kv[1],
+            torch.zeros(2 + m, dtype=torch.int32, device=DEV), torch.zeros(1 << 18, dtype=torch.float32, device=DEV),
+            torch.zeros(64, dtype=torch.int32, device=DEV), 64, n_heads,
+            torch.zeros(m, n_heads * 128, dtype=torch.bfloat16, device=DEV),
+            torch.zeros(m, 8, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("kind", ["t2g128", "q1"])
+def test_decode_loop_tokens_do_not_depend_on_the_self_merging_attention(kind, monkeypatch):
+    """Greedy AR decoding through graphs whose attention merges its own partials (five launches a
+    layer) and through graphs with the separate merge gives the same tokens and logits bits."""
+    from bitmtp_amd import generate
+    from bitmtp_amd.model import BonsaiDecoder, ModelArgs, fused_plan
+    from bitmtp_amd.runtime import GraphAtlas
+    args = ModelArgs(dim=512, n_layers=3, n_heads=4, n_kv_heads=2, ffn_dim=1024, vocab_size=1000,
+                     mask_token_id=999, kernel_kind=kind)
+    model = BonsaiDecoder.random_init(args, seed=31, device=DEV)
+    prompt = np.random.default_rng(6).integers(0, 1000, 70).tolist()
+    runs = {}
+    for flag in ("1", "0"):
+        monkeypatch.setenv("BONSAI_ATTENTION_ONE_LAUNCH", flag)
+        assert (fused_plan(model, 1).attn > 0) == (flag == "1")
+        atlas = GraphAtlas(model, segment_ladder=(128,), threshold=0.9)
+        print(f"[case] AR decode kind={kind} BONSAI_ATTENTION_ONE_LAUNCH={flag}", flush=True)
+        toks, _ = generate.ar_generate(atlas, prompt, max_gen_len=40)
+        runs[flag] = (toks, atlas.workspace.logits[:1].clone())
+        del atlas
+    assert runs["1"][0] == runs["0"][0]
+    assert _same_bits(runs["1"][1], runs["0"][1])
