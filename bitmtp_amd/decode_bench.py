@@ -153,21 +153,27 @@ def run_slot_costs(model_name: str = "1.7b", cache_len: int = 500, device: str =
             row["add_norm_quant_us_per_launch"] = round((base - graph_us(M, role)) / (2 * n_layers + 1), 2)
             ops.actq_lib = saved[3]
             if M <= ops.FUSED_MAX_TOKENS:
-                # the six-launch layer: each fused projection by what it reads and stores, and the
-                # attention that derives q / k itself (two launches)
+                # the fused layer: each projection by what it reads and stores, and the attention
+                # that derives q / k itself and merges its own partials (one launch; two when the
+                # merge is a launch of its own)
                 os.environ["BONSAI_FUSED_STEP"] = "1"
+                plan = mdl.fused_plan(model, M)
+                per_layer = 5 if plan.attn else 6
                 fbase = graph_us(M, role)
-                frow = {"graph_us": round(fbase, 1), "launches": 6 * n_layers + 5}
-                rope_attn = decode_ops.decode_attention_rope
+                frow = {"graph_us": round(fbase, 1), "launches": per_layer * n_layers + 5,
+                        "attention_launches_per_layer": 1 if plan.attn else 2}
+                rope_attn = (decode_ops.decode_attention_rope, decode_ops.decode_attention_rope_parts)
                 decode_ops.decode_attention_rope = lambda *a, **k: None
-                frow["attention_with_rope_us_per_layer_2_launches"] = round((fbase - graph_us(M, role)) / n_layers, 2)
-                decode_ops.decode_attention_rope = rope_attn
-                for label, act_kind, epi in (("qkv_norm_in", ops.ACT_BF16_NORM, ops.EPI_PLAIN),
-                                             ("o_add_out", ops.ACT_INT8, ops.EPI_ADD_SUMSQ),
-                                             ("gate_up_norm_in_silu_out", ops.ACT_BF16_NORM, ops.EPI_SILU_PAIR),
-                                             ("down_amax_in_add_out", ops.ACT_BF16_AMAX, ops.EPI_ADD_SUMSQ)):
-                    def without(w, m, stream, _skip=(act_kind, epi), **kw):
-                        if (kw["act_kind"], kw["epi"]) != _skip:
+                decode_ops.decode_attention_rope_parts = lambda *a, **k: None
+                frow["attention_with_rope_us_per_layer"] = round((fbase - graph_us(M, role)) / n_layers, 2)
+                decode_ops.decode_attention_rope, decode_ops.decode_attention_rope_parts = rope_attn
+                lw0 = model.layers[0]
+                for label, which in (("qkv_norm_in", "wqkv"), ("o_add_out", "wo"),
+                                     ("gate_up_norm_in_silu_out", "w_gu"), ("down_amax_in_add_out", "w_down")):
+                    shape = (getattr(lw0, which).out_features, getattr(lw0, which).in_features)
+
+                    def without(w, m, stream, _skip=shape, **kw):
+                        if (w.out_features, w.in_features) != _skip:
                             saved[4](w, m, stream, **kw)
                     mdl._fused = without
                     n = n_layers - 1 if label == "qkv_norm_in" else n_layers

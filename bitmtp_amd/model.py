@@ -467,9 +467,10 @@ class FusedPlan:
 
 def fused_plan(model: "BonsaiDecoder", m: int) -> Optional[FusedPlan]:
     """How a step of width ``m`` runs its layers: with the residual add + RMSNorm + quantisation
-    and the SiLU * up + quantisation folded into the projections and q / k norm + RoPE into the attention (six
-    launches a layer instead of ten; blocks of one or two tokens), or -- ``None`` -- with the separate producers (wider blocks,
-    shapes the fused kernels do not take, BONSAI_FUSED_STEP=0)."""
+    and the SiLU * up + quantisation folded into the projections, q / k norm + RoPE into the
+    attention and -- ``attn`` > 0 -- the merge of the attention's partials as well (five launches a
+    layer instead of ten; blocks of one or two tokens), or -- ``None`` -- with the separate
+    producers (wider blocks, shapes the fused kernels do not take, BONSAI_FUSED_STEP=0)."""
     if m > ops.FUSED_MAX_TOKENS or os.environ.get("BONSAI_FUSED_STEP", "1") == "0":
         return None
     lw = model.layers[0]
@@ -540,8 +541,9 @@ def enqueue_step(model: BonsaiDecoder, ws: Workspace, io: StepIO, kv: torch.Tens
     torch.index_select(model.embed, 0, io.tokens, out=h_cur)
     for i, lw in enumerate(model.layers):
         if plan is not None:
-            # six launches: the element-wise producers ride in the projections on either side and
-            # the q / k norm + RoPE in the attention;
+            # five launches (six when the attention's merge is a launch of its own): the
+            # element-wise producers ride in the projections on either side, the q / k norm +
+            # RoPE in the attention;
             # h_cur already holds the residual stream including the previous layer's MLP
             if i == 0:
                 check(actq.bonsai_rmsnorm_quant_int8(_vp(h_cur), _vp(lw.input_layernorm), eps,
