@@ -66,6 +66,30 @@ def test_exact_verification_reproduces_ar_at_full_size(full):
     assert st2["decode_tokens"] == 1 + st2["accepted_drafts"] + st2["verifier_bonus_tokens"]
 
 
+def test_ar_tokens_do_not_depend_on_the_layer_form_at_full_size(full, monkeypatch):
+    """Greedy AR decoding at full size through the ten-launch layer, the fused layer with the
+    attention's merge as a launch of its own and the fused layer with the self-merging attention:
+    the same tokens and the same logits bits after the last step."""
+    from bitmtp_amd import generate
+    from bitmtp_amd.runtime import GraphAtlas
+    name, sigma, model, _ = full
+    n_prompt, n_new = (256, 200) if name == "1.7b" else (1000, 120)
+    prompt = np.random.default_rng(29).integers(0, model.args.vocab_size, n_prompt).tolist()
+    runs = []
+    for fused, one_launch in (("0", "1"), ("1", "0"), ("1", "1")):
+        monkeypatch.setenv("BONSAI_FUSED_STEP", fused)
+        monkeypatch.setenv("BONSAI_ATTENTION_ONE_LAUNCH", one_launch)
+        atlas = GraphAtlas(model, segment_ladder=(sigma,), threshold=0.9, roles=("ar",))
+        print(f"[case] {name}: AR {n_new} tokens, BONSAI_FUSED_STEP={fused} "
+              f"BONSAI_ATTENTION_ONE_LAUNCH={one_launch}", flush=True)
+        toks, _ = generate.ar_generate(atlas, prompt, max_gen_len=n_new)
+        runs.append((toks, atlas.workspace.logits[:1].clone()))
+        del atlas
+    for toks, logits in runs[1:]:
+        assert toks == runs[0][0]
+        assert torch.equal(logits.view(torch.int16), runs[0][1].view(torch.int16))
+
+
 def test_graph_replay_equals_eager_at_full_size(full):
     from bitmtp_amd.runtime import GraphAtlas
     name, sigma, model, atlas = full
