@@ -18,7 +18,7 @@ HIP graph so that the Python launch cost is outside the measurement, as in the
 reference's graph-replayed decode.
 
 Beside the headline, `config` carries the rest of the target range on the same timing (one
-graph per figure over >= 512 MB of distinct weights): BASELINE configs[0] (one 6144 x 2048 GEMV
+graph per figure over >= 512 MB of distinct weights): BASELINE.json configs[0] (one 6144 x 2048 GEMV
 at width 1), the 4B-shaped layer (K = 2560, 4096, 9728) grouped and as its four merged
 matrices, the Q1-g128 set of configs[4], both packed lm_heads, and the end-to-end decode runs.
 Every figure names the kernel that was launched (read back from the library, not written here).
@@ -515,7 +515,7 @@ def main() -> int:
         "read_probe_us": per_width[dom]["read_probe_us"],
     }
 
-    # ---- the rest of the target range (BASELINE: T2 K = 2048..9728, Q1 configs[4])
+    # ---- the rest of the target range (BASELINE.json: T2 K = 2048..9728, Q1 configs[4])
     config0 = layer_4b = q1_set = None
     if not args.no_extra:
         from bitmtp_amd import gemv_bench
