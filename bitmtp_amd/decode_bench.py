@@ -3,6 +3,8 @@
     python -m bitmtp_amd.decode_bench --model 1.7b            # 256-token prompt, 512 new
     python -m bitmtp_amd.decode_bench --model 4b --prompt 512 --new 1024
     python -m bitmtp_amd.decode_bench --model 4b --kind q1    # sign weights, bf16 lm_head
+    python -m bitmtp_amd.decode_bench --slot-costs            # what each operator costs inside the captured step
+    python -m bitmtp_amd.decode_bench --attention-sweep       # attention time against the history length
 
 Reports tokens/s by the reference's timing contract (``timed_decode_tokens /
 decode_time``, prefill and the first token excluded; src/bonsai_sft/gpu/fast_generate.py:
@@ -191,6 +193,56 @@ def run_slot_costs(model_name: str = "1.7b", cache_len: int = 500, device: str =
     return out
 
 
+def run_attention_sweep(model_name: str = "1.7b", device: str = "cuda:0", replays: int = 20) -> dict:
+    """Time of the attention (chunk pass + merge, two launches) per layer against the length of
+    the history, for blocks of one and nine rows: a graph of one call per layer over distinct KV
+    buffers (nothing is served from a cache), segment sizes 1024, 4096 and 8192 slots."""
+    from . import decode_ops, runtime
+    args = MODELS[model_name]()
+    n_heads, n_kv, n_layers = args.n_heads, args.n_kv_heads, args.n_layers
+    gen = torch.Generator(device=device)
+    gen.manual_seed(1)
+    rows = []
+    for sigma in (1024, 4096, 8192):
+        slots = sigma + decode_ops.MAX_WIDTH
+        kv = torch.randn(n_layers, 2, n_kv, slots, decode_ops.HEAD_DIM, generator=gen,
+                         device=device).to(torch.bfloat16)
+        for m, role in ((1, "ar"), (9, "verify")):
+            q = torch.randn(m, n_heads, decode_ops.HEAD_DIM, generator=gen, device=device).to(torch.bfloat16)
+            scratch = torch.empty(decode_ops.attention_scratch_bytes(m, n_heads, slots) // 4,
+                                  dtype=torch.float32, device=device)
+            o_q = torch.zeros(m, n_heads * decode_ops.HEAD_DIM, dtype=torch.int8, device=device)
+            o_s = torch.zeros(m, dtype=torch.float32, device=device)
+            for frac in (0.12, 0.45, 0.95):
+                cache_len = int(sigma * frac)
+                meta = torch.tensor(runtime.step_descriptor(role, m, args.block_size, cache_len, 0),
+                                    dtype=torch.int32, device=device)
+
+                def layers():
+                    for layer in range(n_layers):
+                        decode_ops.decode_attention(q, kv[layer, 0], kv[layer, 1], meta, scratch, sigma,
+                                                    out_q=o_q, out_s=o_s)
+                layers()
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    layers()
+                graph.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(replays):
+                    graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) / replays / n_layers * 1e3
+                kv_bytes = 2 * n_kv * (cache_len + m) * decode_ops.HEAD_DIM * 2
+                rows.append({"segment": sigma, "rows": m, "cache_len": cache_len,
+                             "us_per_layer": round(us, 2), "kv_gbps": round(kv_bytes / us / 1e3, 1)})
+        del kv
+    return {"model": model_name, "n_heads": n_heads, "n_kv_heads": n_kv, "attention": rows}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--model", choices=sorted(MODELS), default="1.7b")
@@ -209,9 +261,14 @@ def main() -> None:
     ap.add_argument("--slot-costs", action="store_true",
                     help="instead of tokens/s: the cost of each operator type inside the captured "
                          "step (graphs captured with that operator left out)")
+    ap.add_argument("--attention-sweep", action="store_true",
+                    help="instead of tokens/s: the attention's time per layer against the history length")
     a = ap.parse_args()
     if a.slot_costs:
         print(json.dumps(run_slot_costs(a.model)))
+        return
+    if a.attention_sweep:
+        print(json.dumps(run_attention_sweep(a.model)))
         return
     print(json.dumps(run_decode_bench(a.model, a.prompt, a.new, a.seed, a.repeats,
                                       n_layers=a.layers, kernel_kind=a.kind, head_kind=a.head,
